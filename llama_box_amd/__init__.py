@@ -36,7 +36,8 @@ ROPE_VISION = 24  # mrope with independent sections, pairs (i, i + n_dims) over 
 
 def build(verbose=False):
     """Compile both libraries for gfx950 (hipcc cross-compiles without a GPU)."""
-    r = subprocess.run(["make", "-C", _DIR, "-j8"], capture_output=True, text=True)
+    jobs = os.environ.get("MAX_JOBS", "8")
+    r = subprocess.run(["make", "-C", _DIR, "-j" + (jobs if jobs.isdigit() else "8")], capture_output=True, text=True)
     if verbose or r.returncode != 0:
         print(r.stdout[-4000:])
         print(r.stderr[-4000:])
@@ -153,6 +154,8 @@ _SIGS = {
     "llm_model_synth": (_P, [C.POINTER(HParams), C.c_uint64, _P, _I, _I, _P]), "llm_model_synth_split": (_P, [C.POINTER(HParams), C.c_uint64, _P, _P]), "llm_synth_gguf": (_I, [C.POINTER(HParams), C.c_uint64, _S]),
     "llm_model_synth_layer_split": (_P, [C.POINTER(HParams), C.c_uint64, C.POINTER(_P), _I]),
     "llm_context_new_layer_split": (_P, [_P, C.POINTER(_P), _I, C.POINTER(ContextParams)]), "llm_layer_split_stats": (None, [_P, C.POINTER(C.c_int64)]),
+    "llm_model_load_dir": (_P, [_S, _P, _I]), "llm_model_synth_config": (_P, [_S, C.c_uint64, _P, _I]),
+    "ggml_norm": (TP, [_P, TP, _F]), "ggml_sqr": (TP, [_P, TP]), "ggml_argsort": (TP, [_P, TP, _I]), "ggml_top_k": (TP, [_P, TP, _I]), "ggml_mul_mat_id": (TP, [_P, TP, TP, TP]),
     "llm_model_load": (_P, [_S, _P]), "llm_model_free": (None, [_P]), "llm_model_hparams": (C.POINTER(HParams), [_P]),
     "llm_model_stream_bytes": (C.c_uint64, [_P]), "llm_model_total_bytes": (C.c_uint64, [_P]), "llm_model_tensor": (TP, [_P, _S]),
     "llm_context_new": (_P, [_P, _P, COMPUTE_FN, C.POINTER(ContextParams)]), "llm_context_free": (None, [_P]),

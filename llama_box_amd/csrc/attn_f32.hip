@@ -1,0 +1,275 @@
+// attn_f32.hip — FLASH_ATTN_EXT in 32-bit arithmetic over a cache read in place (f32, bf16 or f16 rows), for ANY head sizes: the
+// query/key size and the value size may differ and need not be 64 or 128.  Scores, soft-max weights and the weighted sum of V are f32
+// from start to end (a cache value is widened exactly; nothing is rounded to 16 bits on the way), so an f32 cache gives true 32-bit
+// attention.  Optional sinks: one extra score per head that takes part in the soft-max denominator and carries no value (src[4] of the op).
+//
+// Two kernels:
+//   k_attn_f32_rows  — one workgroup per (query token, head), its four waves take the cache in interleaved blocks of 64 cells and merge
+//                      their (max, sum, accumulator) through LDS; a block none of whose cells the mask lets through is skipped after
+//                      one 128-byte mask read (attention confined to a window or a chunk touches few blocks).  Decode steps and
+//                      small batches.
+//   k_attn_f32_tile  — prompt batches: a workgroup owns 64 query tokens of one head; K and V blocks of 64 cells are staged through LDS as
+//                      f32 once per workgroup and every wave runs 16 of the queries against them (a lane owns one cell for the scores
+//                      and one or more value columns for the sum); blocks the mask hides from all 64 queries are skipped.
+#include <algorithm>
+
+#include "dev_util.h"
+#include "kernels.h"
+
+namespace mi355x {
+
+template <int T> __device__ __forceinline__ float kv_ld(const char * __restrict__ row, const int i) {
+    if constexpr (T == GGML_TYPE_F32) return ((const float *) row)[i];
+    else if constexpr (T == GGML_TYPE_BF16) return __uint_as_float((uint32_t) ((const uint16_t *) row)[i] << 16);
+    else return h2f(((const uint16_t *) row)[i]);
+}
+
+__device__ __forceinline__ float wave_max_f(float v) {
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ float wave_sum_f(float v) {
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+constexpr int ATTN_F32_MAX_D = 256;   // largest head size (query/key or value)
+constexpr float ATTN_F32_LOW = -1e30f;  // "no score yet": finite, so that differences of maxima never give NaN
+
+// mask element -> additive term (f16 or f32 mask rows; -inf hides the cell)
+__device__ __forceinline__ float mask_ld(const char * __restrict__ mrow, const int mtype, const int64_t j) {
+    return mtype == GGML_TYPE_F16 ? h2f(((const uint16_t *) mrow)[j]) : ((const float *) mrow)[j];
+}
+
+template <int KT, int VT>
+__global__ void __launch_bounds__(256) k_attn_f32_rows(const tdesc q, const tdesc k, const tdesc v, const tdesc mask, const int has_mask, const float * __restrict__ sinks,
+                                                       const tdesc dst, const float scale) {
+    __shared__ float qs[ATTN_F32_MAX_D];
+    __shared__ float part_acc[4][ATTN_F32_MAX_D];
+    __shared__ float part_m[4], part_l[4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t t = blockIdx.x, h = blockIdx.y;
+    const int DK = (int) q.ne[0], DV = (int) v.ne[0];
+    const int64_t n_kv = k.ne[1];
+    const int64_t g = h / (q.ne[2] / k.ne[2]);
+    const char * qrow = q.data + t * q.nb[1] + h * q.nb[2];
+    for (int i = threadIdx.x; i < DK; i += 256) qs[i] = ((const float *) qrow)[i];
+    __syncthreads();
+    const char * mrow = has_mask ? mask.data + t * mask.nb[1] : nullptr;
+    const char * kbase = k.data + g * k.nb[2];
+    const char * vbase = v.data + g * v.nb[2];
+    float m = ATTN_F32_LOW, l = 0.0f;
+    if (sinks && wave == 0) { m = sinks[h]; l = 1.0f; }  // the sink: exp(sink - m) = 1 in the denominator, nothing in the numerator
+    float acc[ATTN_F32_MAX_D / 64];
+#pragma unroll
+    for (int r = 0; r < ATTN_F32_MAX_D / 64; ++r) acc[r] = 0.0f;
+    for (int64_t j0 = (int64_t) wave * 64; j0 < n_kv; j0 += 256) {
+        const int64_t j = j0 + lane;
+        float mv = -INFINITY;
+        if (j < n_kv) mv = has_mask ? mask_ld(mrow, mask.type, j) : 0.0f;
+        const bool vis = mv > -INFINITY;
+        const uint64_t live = __ballot(vis);
+        if (!live) continue;
+        float s = -INFINITY;
+        if (vis) {
+            const char * krow = kbase + j * k.nb[1];
+            float d = 0.0f;
+            for (int i = 0; i < DK; ++i) d = fmaf(qs[i], kv_ld<KT>(krow, i), d);
+            s = d * scale + mv;
+        }
+        const float m_new = fmaxf(m, wave_max_f(s));
+        const float p = vis ? expf(s - m_new) : 0.0f;
+        const float corr = expf(m - m_new);
+        l = l * corr + wave_sum_f(p);
+        m = m_new;
+#pragma unroll
+        for (int r = 0; r < ATTN_F32_MAX_D / 64; ++r) acc[r] *= corr;
+        uint64_t todo = live;
+        while (todo) {
+            const int jj = __builtin_ctzll(todo);
+            todo &= todo - 1;
+            const float pj = __shfl(p, jj, 64);
+            const char * vrow = vbase + (j0 + jj) * v.nb[1];
+#pragma unroll
+            for (int r = 0; r < ATTN_F32_MAX_D / 64; ++r) {
+                const int dcol = lane + 64 * r;
+                if (dcol < DV) acc[r] = fmaf(pj, kv_ld<VT>(vrow, dcol), acc[r]);
+            }
+        }
+    }
+    if (lane == 0) { part_m[wave] = m; part_l[wave] = l; }
+#pragma unroll
+    for (int r = 0; r < ATTN_F32_MAX_D / 64; ++r) {
+        const int dcol = lane + 64 * r;
+        if (dcol < DV) part_acc[wave][dcol] = acc[r];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    float M = part_m[0];
+    for (int w = 1; w < 4; ++w) M = fmaxf(M, part_m[w]);
+    float L = 0.0f, cw[4];
+    for (int w = 0; w < 4; ++w) { cw[w] = expf(part_m[w] - M); L += part_l[w] * cw[w]; }
+    const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+    float * out = (float *) (dst.data + h * dst.nb[1] + t * dst.nb[2]);
+    for (int dcol = lane; dcol < DV; dcol += 64) {
+        float o = 0.0f;
+        for (int w = 0; w < 4; ++w) o += part_acc[w][dcol] * cw[w];
+        out[dcol] = o * inv;
+    }
+}
+
+// prompt batches: 64 query tokens x one head per workgroup; K / V blocks of 64 cells staged in LDS as f32
+template <int KT, int VT, int DKP, int DVP>   // DKP / DVP: head sizes rounded up to a multiple of 32 / 64 (LDS row lengths)
+__global__ void __launch_bounds__(256) k_attn_f32_tile(const tdesc q, const tdesc k, const tdesc v, const tdesc mask, const float * __restrict__ sinks, const tdesc dst,
+                                                       const float scale) {
+    constexpr int QT = 64, KB = 64, QW = QT / 4;  // queries per workgroup, cells per block, queries per wave
+    constexpr int KS = DKP + 1;                   // K row stride in LDS (odd: lanes that read column i of 64 different rows hit 64 different banks)
+    extern __shared__ float lds[];
+    float * Ks = lds;                    // [KB][KS]
+    float * Vs = Ks + KB * KS;           // [KB][DVP]
+    float * Qs = Vs + KB * DVP;          // [QT][DKP]
+    __shared__ int blk_live;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t t0 = (int64_t) blockIdx.x * QT, h = blockIdx.y;
+    const int DK = (int) q.ne[0], DV = (int) v.ne[0];
+    const int64_t n_kv = k.ne[1], n_q = q.ne[1];
+    const int64_t g = h / (q.ne[2] / k.ne[2]);
+    const char * kbase = k.data + g * k.nb[2];
+    const char * vbase = v.data + g * v.nb[2];
+    for (int e = threadIdx.x; e < QT * DKP; e += 256) {
+        const int qi = e / DKP, i = e % DKP;
+        const int64_t t = t0 + qi;
+        Qs[e] = (t < n_q && i < DK) ? ((const float *) (q.data + t * q.nb[1] + h * q.nb[2]))[i] : 0.0f;
+    }
+    float m[QW], l[QW], acc[QW][DVP / 64];
+#pragma unroll
+    for (int qi = 0; qi < QW; ++qi) {
+        m[qi] = sinks ? sinks[h] : ATTN_F32_LOW;
+        l[qi] = sinks ? 1.0f : 0.0f;
+#pragma unroll
+        for (int r = 0; r < DVP / 64; ++r) acc[qi][r] = 0.0f;
+    }
+    for (int64_t j0 = 0; j0 < n_kv; j0 += KB) {
+        // does any of the 64 queries see any of the 64 cells?  (one mask element per thread and query row quarter)
+        __syncthreads();
+        if (threadIdx.x == 0) blk_live = 0;
+        __syncthreads();
+        {
+            bool any = false;
+            for (int qi = wave; qi < QT; qi += 4) {
+                const int64_t t = t0 + qi, j = j0 + lane;
+                if (t < n_q && j < n_kv) any = any || mask_ld(mask.data + t * mask.nb[1], mask.type, j) > -INFINITY;
+            }
+            if (__ballot(any) && lane == 0) blk_live = 1;
+        }
+        __syncthreads();
+        if (!blk_live) continue;
+        for (int e = threadIdx.x; e < KB * DKP; e += 256) {
+            const int r = e / DKP, i = e % DKP;
+            const int64_t j = j0 + r;
+            Ks[r * KS + i] = (j < n_kv && i < DK) ? kv_ld<KT>(kbase + j * k.nb[1], i) : 0.0f;
+        }
+        for (int e = threadIdx.x; e < KB * DVP; e += 256) {
+            const int r = e / DVP, i = e % DVP;
+            const int64_t j = j0 + r;
+            Vs[e] = (j < n_kv && i < DV) ? kv_ld<VT>(vbase + j * v.nb[1], i) : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int qi = 0; qi < QW; ++qi) {
+            const int ql = wave * QW + qi;
+            const int64_t t = t0 + ql, j = j0 + lane;
+            float mv = -INFINITY;
+            if (t < n_q && j < n_kv) mv = mask_ld(mask.data + t * mask.nb[1], mask.type, j);
+            const bool vis = mv > -INFINITY;
+            const uint64_t live = __ballot(vis);
+            if (!live) continue;
+            float d = 0.0f;
+            const float * qr = Qs + ql * DKP;
+            const float * kr = Ks + lane * KS;
+            for (int i = 0; i < DK; ++i) d = fmaf(qr[i], kr[i], d);
+            const float s = vis ? d * scale + mv : -INFINITY;
+            const float m_new = fmaxf(m[qi], wave_max_f(s));
+            const float p = vis ? expf(s - m_new) : 0.0f;
+            const float corr = expf(m[qi] - m_new);
+            l[qi] = l[qi] * corr + wave_sum_f(p);
+            m[qi] = m_new;
+#pragma unroll
+            for (int r = 0; r < DVP / 64; ++r) acc[qi][r] *= corr;
+            uint64_t todo = live;
+            while (todo) {
+                const int jj = __builtin_ctzll(todo);
+                todo &= todo - 1;
+                const float pj = __shfl(p, jj, 64);
+#pragma unroll
+                for (int r = 0; r < DVP / 64; ++r) acc[qi][r] = fmaf(pj, Vs[jj * DVP + lane + 64 * r], acc[qi][r]);
+            }
+        }
+    }
+#pragma unroll
+    for (int qi = 0; qi < QW; ++qi) {
+        const int64_t t = t0 + wave * QW + qi;
+        if (t >= n_q) continue;
+        const float inv = l[qi] > 0.0f ? 1.0f / l[qi] : 0.0f;
+        float * out = (float *) (dst.data + h * dst.nb[1] + t * dst.nb[2]);
+#pragma unroll
+        for (int r = 0; r < DVP / 64; ++r) {
+            const int dcol = lane + 64 * r;
+            if (dcol < DV) out[dcol] = acc[qi][r] * inv;
+        }
+    }
+}
+
+static bool attn_f32_type_ok(int t) { return t == GGML_TYPE_F32 || t == GGML_TYPE_BF16 || t == GGML_TYPE_F16; }
+
+// may launch_attn_f32 serve this op?  q f32 [DK, n_q, H], k [DK, n_kv, G], v [DV, n_kv, G] of one type each, rows contiguous, one batch
+bool attn_f32_applies(const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const tdesc & dst) {
+    if (q.type != GGML_TYPE_F32 || dst.type != GGML_TYPE_F32 || !attn_f32_type_ok(k.type) || !attn_f32_type_ok(v.type)) return false;
+    if (q.ne[0] != k.ne[0] || k.ne[1] != v.ne[1] || k.ne[2] != v.ne[2] || k.ne[2] <= 0 || q.ne[2] % k.ne[2] != 0) return false;
+    if (q.ne[0] < 1 || q.ne[0] > ATTN_F32_MAX_D || v.ne[0] < 1 || v.ne[0] > ATTN_F32_MAX_D) return false;
+    if (q.ne[3] != 1 || k.ne[3] != 1 || v.ne[3] != 1) return false;
+    if (q.nb[0] != 4 || dst.nb[0] != 4 || k.nb[0] != (k.type == GGML_TYPE_F32 ? 4 : 2) || v.nb[0] != (v.type == GGML_TYPE_F32 ? 4 : 2)) return false;
+    if (dst.ne[0] != v.ne[0] || dst.ne[1] != q.ne[2] || dst.ne[2] != q.ne[1]) return false;
+    if (mask && ((mask->type != GGML_TYPE_F16 && mask->type != GGML_TYPE_F32) || mask->ne[0] < k.ne[1] || mask->ne[1] < q.ne[1] || mask->ne[2] != 1 || mask->ne[3] != 1)) return false;
+    return true;
+}
+
+template <int KT, int VT>
+static void attn_f32_launch_t(hipStream_t s, const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const float * sinks, const tdesc & dst, float scale) {
+    const int64_t n_q = q.ne[1], H = q.ne[2];
+    const int DK = (int) q.ne[0], DV = (int) v.ne[0];
+    // the tile kernel: batches of 32 queries and more under a mask, head sizes up to 128 (its LDS: 64 cells of K and V plus 64 queries as f32)
+    if (mask && n_q >= 32 && DK <= 128 && DV <= 128) {
+        const dim3 grid((unsigned) ((n_q + 63) / 64), (unsigned) H);
+        auto go = [&](auto kern, int dkp, int dvp) {
+            const size_t lds = ((size_t) 64 * (dkp + 1) + (size_t) 64 * dvp + (size_t) 64 * dkp) * sizeof(float);
+            hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, q, k, v, *mask, sinks, dst, scale);
+        };
+        const bool k64 = DK <= 64, v64 = DV <= 64;
+        if (k64 && v64) go(k_attn_f32_tile<KT, VT, 64, 64>, 64, 64);
+        else if (k64) go(k_attn_f32_tile<KT, VT, 64, 128>, 64, 128);
+        else if (v64) go(k_attn_f32_tile<KT, VT, 128, 64>, 128, 64);
+        else go(k_attn_f32_tile<KT, VT, 128, 128>, 128, 128);
+        return;
+    }
+    hipLaunchKernelGGL((k_attn_f32_rows<KT, VT>), dim3((unsigned) n_q, (unsigned) H), dim3(256), 0, s, q, k, v, mask ? *mask : q, mask ? 1 : 0, sinks, dst, scale);
+}
+
+void launch_attn_f32(hipStream_t s, const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const float * sinks, const tdesc & dst, float scale) {
+    if (q.ne[1] == 0 || q.ne[2] == 0) return;
+#define MI_ATTN_F32_CASE(KT, VT) if (k.type == KT && v.type == VT) { attn_f32_launch_t<KT, VT>(s, q, k, v, mask, sinks, dst, scale); return; }
+    MI_ATTN_F32_CASE(GGML_TYPE_F32, GGML_TYPE_F32)
+    MI_ATTN_F32_CASE(GGML_TYPE_BF16, GGML_TYPE_BF16)
+    MI_ATTN_F32_CASE(GGML_TYPE_F16, GGML_TYPE_F16)
+    MI_ATTN_F32_CASE(GGML_TYPE_F32, GGML_TYPE_BF16)
+    MI_ATTN_F32_CASE(GGML_TYPE_BF16, GGML_TYPE_F32)
+    MI_ATTN_F32_CASE(GGML_TYPE_F32, GGML_TYPE_F16)
+    MI_ATTN_F32_CASE(GGML_TYPE_F16, GGML_TYPE_F32)
+    MI_ATTN_F32_CASE(GGML_TYPE_BF16, GGML_TYPE_F16)
+    MI_ATTN_F32_CASE(GGML_TYPE_F16, GGML_TYPE_BF16)
+#undef MI_ATTN_F32_CASE
+}
+
+MI_TU_TOUCH(attn_f32)
+
+}  // namespace mi355x

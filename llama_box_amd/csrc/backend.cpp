@@ -901,6 +901,7 @@ static int64_t api_get_stat(ggml_backend_t be, const char * key) {
     if (k == "kernel_downloads") return c->st.kernel_downloads;
     if (k == "kv_image_nodes") return c->st.kv_image_nodes;
     if (k == "kv_native_nodes") return c->st.kv_native_nodes;
+    if (k == "attn_f32_nodes") return c->st.attn_f32_nodes;
     if (k == "graph_key_host_ns") return c->st.graph_key_host_ns;
     if (k == "graph_compute_host_ns") return c->st.graph_compute_host_ns;
     if (k == "graph_key_fast_hits") return c->st.graph_key_fast_hits;
@@ -1033,6 +1034,7 @@ static bool op_numbering_matches_host() {
         {GGML_OP_CPY, "CPY"}, {GGML_OP_CONT, "CONT"}, {GGML_OP_RESHAPE, "RESHAPE"}, {GGML_OP_VIEW, "VIEW"}, {GGML_OP_PERMUTE, "PERMUTE"},
         {GGML_OP_TRANSPOSE, "TRANSPOSE"}, {GGML_OP_GET_ROWS, "GET_ROWS"}, {GGML_OP_SET_ROWS, "SET_ROWS"}, {GGML_OP_SOFT_MAX, "SOFT_MAX"},
         {GGML_OP_ROPE, "ROPE"}, {GGML_OP_FLASH_ATTN_EXT, "FLASH_ATTN_EXT"}, {GGML_OP_UNARY, "UNARY"}, {GGML_OP_GLU, "GLU"},
+        {GGML_OP_NORM, "NORM"}, {GGML_OP_SQR, "SQR"}, {GGML_OP_ARGSORT, "ARGSORT"},
     };
     bool ok = true;
     for (const auto & e : k_expect) {

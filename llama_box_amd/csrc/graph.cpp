@@ -58,12 +58,30 @@ static bool mm_cache_image_ok(const ggml_tensor * op) {
 // which attention path serves this FLASH_ATTN_EXT node: 0 none (the host keeps it on the CPU backend), 1 the f16 kernels on the cache views in place,
 // 2 the lane-parallel kernel on block_q8_0 K / V, 3 the f16 kernels on an f16 IMAGE of whichever of K / V is kept in another type (kv_types.hip:
 // -ctk / -ctv q4_0, q4_1, q5_0, q5_1, iq4_nl, bf16, f32, mixed pairs, and q8_0 shapes route 2 does not take)
+// route 4: the 32-bit kernel over f32 / bf16 / f16 rows read in place (attn_f32.hip) — a cache kept in f32 or bf16 (its values are used as
+// they are, not through an f16 image), head sizes other than 64 / 128, a value size that differs from the key size
+static bool fa_f32_route(const ggml_tensor * op) {
+    const ggml_tensor * a = op->src[0];
+    const ggml_tensor * k = op->src[1];
+    const ggml_tensor * v = op->src[2];
+    const ggml_tensor * m = op->src[3];
+    if (ggml_abi_op_param_f32(op, 1) != 0.0f || ggml_abi_op_param_f32(op, 2) != 0.0f) return false;  // no ALiBi slopes, no soft-capping there
+    if (op->src[4] && (op->src[4]->type != GGML_TYPE_F32 || ggml_abi_nelements(op->src[4]) < a->ne[2])) return false;
+    const tdesc md = m ? TD(m) : TD(a);
+    return attn_f32_applies(TD(a), TD(k), TD(v), m ? &md : nullptr, TD(op));
+}
 static int fa_route(const ggml_tensor * op) {
     const ggml_tensor * a = op->src[0];
     const ggml_tensor * k = op->src[1];
     const ggml_tensor * v = op->src[2];
     const ggml_tensor * m = op->src[3];
     if (!a || !k || !v || a->type != GGML_TYPE_F32) return 0;
+    {
+        const bool wide_k = k->type == GGML_TYPE_F32 || k->type == GGML_TYPE_BF16, wide_v = v->type == GGML_TYPE_F32 || v->type == GGML_TYPE_BF16;
+        const bool plain = (wide_k || k->type == GGML_TYPE_F16) && (wide_v || v->type == GGML_TYPE_F16);
+        const bool odd_shape = k->ne[0] != v->ne[0] || (k->ne[0] != 64 && k->ne[0] != 128);
+        if (plain && ((wide_k && wide_v) || odd_shape) && fa_f32_route(op)) return 4;
+    }
     if (k->type == GGML_TYPE_Q8_0 && v->type == GGML_TYPE_Q8_0) {
         // quantised KV cache: served by the lane-parallel kernel (head_dim 128, 1 .. 8 query heads per KV head, no soft-capping / ALiBi)
         const int64_t g = k->ne[2] ? a->ne[2] / k->ne[2] : 0;
@@ -108,6 +126,7 @@ bool supports_op(const ggml_tensor * op) {
             if (!a || !b || b->type != GGML_TYPE_F32 || op->type != GGML_TYPE_F32 || !ggml_abi_is_contiguous(op)) return false;
             if (buffer_is_split(a->buffer)) return split_mul_mat_supported(op);  // -sm row weights: every device computes its rows (split.cpp)
             if (mm_cache_image_ok(op)) return true;
+            if (a->type == GGML_TYPE_BF16) return a->nb[0] == 2 && b->nb[0] == 4;  // a model's bf16 matrices: src1 rounded to bf16, f32 accumulation (mmf.hip)
             if (is_quant(a->type)) {
                 return a->ne[2] == 1 && a->ne[3] == 1 && rows_contig(a) && b->nb[0] == 4 && a->ne[0] % ggml_abi_blck_size(a->type) == 0;
             }
@@ -119,12 +138,23 @@ bool supports_op(const ggml_tensor * op) {
         case GGML_OP_SCALE:
             return is_f32_contig(a) && is_f32_contig(op);
         case GGML_OP_RMS_NORM:
+        case GGML_OP_NORM:
             return a->type == GGML_TYPE_F32 && a->nb[0] == 4 && op->nb[0] == 4;
         case GGML_OP_UNARY: {
             const int u = op->op_params[0];
             const bool ok = u == GGML_UNARY_OP_SILU || u == GGML_UNARY_OP_RELU || u == GGML_UNARY_OP_NEG || u == GGML_UNARY_OP_EXP ||
-                            u == GGML_UNARY_OP_TANH || u == GGML_UNARY_OP_SIGMOID;
+                            u == GGML_UNARY_OP_TANH || u == GGML_UNARY_OP_SIGMOID || u == GGML_UNARY_OP_GELU_ERF || u == GGML_UNARY_OP_GELU;
             return ok && is_f32_contig(a) && is_f32_contig(op);
+        }
+        case GGML_OP_SQR:
+            return is_f32_contig(a) && is_f32_contig(op);
+        case GGML_OP_ARGSORT:
+            return a->type == GGML_TYPE_F32 && a->nb[0] == 4 && op->type == GGML_TYPE_I32 && op->nb[0] == 4 && a->ne[0] <= 65536;
+        case GGML_OP_MUL_MAT_ID: {
+            const ggml_tensor * ids = op->src[2];
+            if (!a || !b || !ids || b->type != GGML_TYPE_F32 || op->type != GGML_TYPE_F32 || ids->type != GGML_TYPE_I32 || !ggml_abi_is_contiguous(op)) return false;
+            if (a->type != GGML_TYPE_F32 && a->type != GGML_TYPE_F16 && a->type != GGML_TYPE_BF16) return false;
+            return a->nb[0] == ggml_abi_type_size(a->type) && b->nb[0] == 4 && a->ne[3] == 1 && b->ne[3] == 1 && (b->ne[1] == 1 || b->ne[1] == ids->ne[0]) && ids->ne[1] == b->ne[2];
         }
         case GGML_OP_GLU:
             return op->op_params[0] == GGML_GLU_OP_SWIGLU && a->type == GGML_TYPE_F32 && a->nb[0] == 4 && (!b || (b->type == GGML_TYPE_F32 && b->nb[0] == 4)) &&
@@ -140,8 +170,10 @@ bool supports_op(const ggml_tensor * op) {
         }
         case GGML_OP_GET_ROWS:
             return b->type == GGML_TYPE_I32 && op->type == GGML_TYPE_F32 && rows_contig(a) && op->nb[0] == 4 &&
-                   (is_quant(a->type) || a->type == GGML_TYPE_F16 || a->type == GGML_TYPE_F32);
+                   (is_quant(a->type) || a->type == GGML_TYPE_F16 || a->type == GGML_TYPE_F32 || a->type == GGML_TYPE_BF16);
         case GGML_OP_SET_ROWS:
+            if (op->type == GGML_TYPE_BF16 && (a->ne[0] % 32) != 0)  // bf16 rows that are not whole groups of 32 values: the element-wise form (ops.hip)
+                return a->type == GGML_TYPE_F32 && b->type == GGML_TYPE_I64 && a->nb[0] == 4 && op->nb[0] == 2;
             if (kv_store_type(op->type))  // a cache row in q4_0 / q4_1 / q5_0 / q5_1 / iq4_nl / bf16: the type's from_float per block of 32 (kv_types.hip)
                 return a->type == GGML_TYPE_F32 && b->type == GGML_TYPE_I64 && a->nb[0] == 4 && (a->ne[0] % 32) == 0 && (a->nb[1] % 16) == 0 && (a->nb[2] % 16) == 0 && (a->nb[3] % 16) == 0 &&
                        op->nb[0] == ggml_abi_type_size(op->type);
@@ -229,6 +261,10 @@ static ws_plan plan_ws(backend_ctx * c, const ggml_cgraph * g) {
             // (K.q of a prompt micro-batch on the non-flash path: statistics + partial records of the two-pass matrix-core form)
             if (c->opt.attn_nf && n->src[1]->type == GGML_TYPE_F32 && n->src[1]->ne[1] >= fattn_mma_min_q() && n->src[0]->ne[0] == 128 && n->src[1]->ne[3] == 1)
                 p.aux_bytes = std::max(p.aux_bytes, attn_nf_mma_ws_bytes(TD(n->src[1]), fattn_mma_pick_splits(TD(n->src[1]), TD(n->src[0]))));
+        } else if (n->op == GGML_OP_MUL_MAT_ID && n->src[2]) {
+            p.aux_bytes = std::max(p.aux_bytes, mul_mat_id_workspace_bytes(TD(n->src[0]), TD(n->src[2])));
+        } else if (n->op == GGML_OP_FLASH_ATTN_EXT && fa_route(n) == 4) {
+            continue;  // the 32-bit kernel keeps its running sums on chip
         } else if (n->op == GGML_OP_FLASH_ATTN_EXT) {
             const tdesc q = TD(n->src[0]), k = TD(n->src[1]), v = TD(n->src[2]);
             // (both forms a 33+-token batch may take — matrix-core tiles or, for a mask known to be sparse, position lists — fit this)
@@ -345,6 +381,9 @@ struct exec_state {
     int ss_n = 0;
     // merged Q/K/V projections whose split-K partial products are summed by the rope + cache-store kernel at node `node`
     struct { int node = -1, n = 0, ks = 0, M = 0; mmq_mat_desc mats[3]; const ggml_tensor * dst[3]; const float * part = nullptr; } rs_sk;
+    // the MUL_MAT_ID that last left per-expert column lists in the scratch area: node index and the ids tensor they were made from
+    int moe_node = -1;
+    const ggml_tensor * moe_ids = nullptr;
 };
 
 // Number of readers of t.  A backend is handed ONE split of the host's graph (ggml_backend_sched: ggml_graph_view of the full
@@ -1867,10 +1906,71 @@ static int run_node(exec_state & st, int i) {
             launch_scale(s, TD(a), TD(n), ggml_abi_op_param_f32(n, 0), ggml_abi_op_param_f32(n, 1));
             c->st.kernel_launches++;
             return 1;
-        case GGML_OP_UNARY:
+        case GGML_OP_UNARY: {
+            // RELU -> SQR (the squared-ReLU activation): one pass writing the SQR's output
+            ggml_tensor * sq = next(1);
+            if (fuse && n->op_params[0] == GGML_UNARY_OP_RELU && sq && sq->op == GGML_OP_SQR && sq->src[0] == n && single_use(st, n) && is_f32_contig(sq) && same_shape(sq, n)) {
+                launch_unary(s, MI_UNARY_RELU_SQR, TD(a), TD(sq));
+                c->st.kernel_launches++;
+                c->st.fused_nodes++;
+                return 2;
+            }
             launch_unary(s, n->op_params[0], TD(a), TD(n));
             c->st.kernel_launches++;
             return 1;
+        }
+        case GGML_OP_SQR:
+            launch_unary(s, MI_UNARY_SQR, TD(a), TD(n));
+            c->st.kernel_launches++;
+            return 1;
+        case GGML_OP_ARGSORT:
+            launch_argsort(s, TD(a), TD(n), n->op_params[0] == 1 ? 1 : 0);
+            c->st.kernel_launches++;
+            return 1;
+        case GGML_OP_NORM: {
+            // NORM -> MUL(norm, w) [-> ADD(.., residual)]: one kernel writing the last node's output
+            ggml_tensor * m = next(1);
+            if (fuse && m && m->op == GGML_OP_MUL && single_use(st, n) && m->type == GGML_TYPE_F32 && m->nb[0] == 4 && same_shape(m, n)) {
+                const ggml_tensor * w = m->src[0] == n ? m->src[1] : (m->src[1] == n ? m->src[0] : nullptr);
+                if (w && w->type == GGML_TYPE_F32 && ggml_abi_is_contiguous(w) && w->ne[0] == n->ne[0] && ggml_abi_nelements(w) == w->ne[0]) {
+                    ggml_tensor * ad = next(2);
+                    const ggml_tensor * res = (ad && ad->op == GGML_OP_ADD && single_use(st, m) && ad->type == GGML_TYPE_F32 && ad->nb[0] == 4 && same_shape(ad, m))
+                                                  ? (ad->src[0] == m ? ad->src[1] : (ad->src[1] == m ? ad->src[0] : nullptr)) : nullptr;
+                    if (res && res->type == GGML_TYPE_F32 && res->nb[0] == 4 && same_shape(res, m) && !(ranges_overlap(ad, a) && ad->data != a->data)) {
+                        const tdesc rd = TD(res);
+                        timed_scope ts(c, "layer_norm_mul_add", (double) ggml_abi_nbytes(a) * 3);
+                        launch_layer_norm(s, TD(a), TD(ad), ggml_abi_op_param_f32(n, 0), (const float *) w->data, &rd);
+                        c->st.kernel_launches++;
+                        c->st.fused_nodes += 2;
+                        return 3;
+                    }
+                    timed_scope ts(c, "layer_norm_mul", (double) ggml_abi_nbytes(a) * 2);
+                    launch_layer_norm(s, TD(a), TD(m), ggml_abi_op_param_f32(n, 0), (const float *) w->data, nullptr);
+                    c->st.kernel_launches++;
+                    c->st.fused_nodes++;
+                    return 2;
+                }
+            }
+            timed_scope ts(c, "layer_norm", (double) ggml_abi_nbytes(a) * 2);
+            launch_layer_norm(s, TD(a), TD(n), ggml_abi_op_param_f32(n, 0), nullptr, nullptr);
+            c->st.kernel_launches++;
+            return 1;
+        }
+        case GGML_OP_MUL_MAT_ID: {
+            const ggml_tensor * ids = n->src[2];
+            // the down projection of a mixture-of-experts block reads the same ids as its up projection: the per-expert column lists are made once
+            // (valid only while nothing but element-wise nodes ran in between: they do not touch the scratch area)
+            bool valid = st.moe_ids == ids && st.moe_node >= 0 && i - st.moe_node <= 6 && g->nodes[st.moe_node]->src[0]->ne[2] == a->ne[2];
+            for (int k = st.moe_node + 1; valid && k < i; ++k) valid = is_view_op(g->nodes[k]) || g->nodes[k]->op == GGML_OP_UNARY || g->nodes[k]->op == GGML_OP_SQR;
+            const size_t need = mul_mat_id_workspace_bytes(TD(a), TD(ids));
+            void * ws = (c->ws && st.aux_off + need <= c->ws_size) ? (char *) c->ws + st.aux_off : nullptr;
+            timed_scope ts(c, "mul_mat_id", (double) ggml_abi_nbytes(a) / (double) std::max<int64_t>(1, a->ne[2]) * (double) std::min<int64_t>(a->ne[2], ggml_abi_nelements(ids)));
+            launch_mul_mat_id(s, TD(a), TD(b), TD(ids), TD(n), ws, ws ? c->ws_size - st.aux_off : 0, valid && ws);
+            st.moe_ids = ws ? ids : nullptr;
+            st.moe_node = i;
+            c->st.kernel_launches++;
+            return 1;
+        }
         case GGML_OP_GLU: {
             const tdesc bd = b ? TD(b) : TD(a);
             if (fuse && c->opt.prologue && ggml_abi_nrows(n) > 1 && (a->nb[1] % 16) == 0 && (!b || (b->nb[1] % 16) == 0) && !(((uintptr_t) a->data) & 15) &&
@@ -1984,7 +2084,7 @@ static int run_node(exec_state & st, int i) {
         case GGML_OP_SET_ROWS: {
             timed_scope ts(c, "set_rows", (double) ggml_abi_nbytes(a));
             if (n->type == GGML_TYPE_Q8_0) launch_set_rows_q8_0(s, TD(a), TD(b), TD(n));
-            else if (kv_store_type(n->type)) {
+            else if (kv_store_type(n->type) && !(n->type == GGML_TYPE_BF16 && (a->ne[0] % 32) != 0)) {
                 // K and V rows of a step go into their caches through the same indices: SET_ROWS(k), [views], SET_ROWS(v) as ONE launch
                 int j = i + 1;
                 while (j < g->n_nodes && (st.done[j] || is_view_op(g->nodes[j]))) ++j;
@@ -2086,6 +2186,14 @@ static int run_node(exec_state & st, int i) {
             p.logit_softcap = ggml_abi_op_param_f32(n, 2);
             const tdesc qd = TD(a);
             tdesc kd = TD(k), vd = TD(v);
+            if (fa_route(n) == 4) {
+                const tdesc md4 = m ? TD(m) : qd;
+                timed_scope ts(c, "attn_f32", (double) ggml_abi_nbytes(k) + (double) ggml_abi_nbytes(v));
+                launch_attn_f32(s, qd, kd, vd, m ? &md4 : nullptr, n->src[4] ? (const float *) n->src[4]->data : nullptr, TD(n), p.scale);
+                c->st.kernel_launches++;
+                c->st.attn_f32_nodes++;
+                return 1;
+            }
             bool imaged = fa_route(n) == 3;
             bool native_kv = false;
             if (imaged) {  // decode-sized batches at the lane-parallel kernel's shapes read the cache IN PLACE (fattn.hip: the DQ form); everything else through the image

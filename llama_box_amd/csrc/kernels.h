@@ -161,6 +161,13 @@ void launch_qkv(hipStream_t s, const qkv_args & a, int type_a, int type_b);
 // src1 rounded to f16 first when src0 is f16 (ggml-cpu vec_dot_type semantics)
 void launch_mul_mat_f(hipStream_t s, const tdesc & src0, const tdesc & src1, const tdesc & dst, float * ws = nullptr, size_t ws_bytes = 0);  // ws: scratch for K-split partial tiles
 size_t mul_mat_f_workspace_bytes(const tdesc & src0, const tdesc & src1);
+// MUL_MAT_ID: as [K, N, n_expert] (f32 / f16 / bf16), b [K, 1 or n_used, T] f32, ids [n_used, T] i32 -> d [N, n_used, T].  ws: scratch for the
+// per-expert column lists of the batched form; lists_valid: an earlier call left the lists of these same ids there
+size_t mul_mat_id_workspace_bytes(const tdesc & as, const tdesc & ids);
+void launch_mul_mat_id(hipStream_t s, const tdesc & as, const tdesc & b, const tdesc & ids, const tdesc & d, void * ws, size_t ws_bytes, bool lists_valid);
+// FLASH_ATTN_EXT in 32-bit arithmetic over f32 / bf16 / f16 K and V read in place, any head sizes up to 256, K and V sizes independent (attn_f32.hip)
+bool attn_f32_applies(const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const tdesc & dst);
+void launch_attn_f32(hipStream_t s, const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const float * sinks, const tdesc & dst, float scale);
 // ---- non-flash attention chain of a small batch over position lists (attn_nf.hip)
 size_t attn_nf_list_scratch_bytes(const tdesc & q, const tdesc & k, int * dq_out);
 bool launch_attn_nf_list(hipStream_t s, const tdesc & q, const tdesc & k, const tdesc & v, const tdesc & mask, const tdesc & dst, const int * lists, int list_stride,
@@ -217,6 +224,11 @@ void launch_mmq(hipStream_t s, int type, const uint8_t * W, int64_t w_nb1, int K
 
 // ---- element-wise / normalisation / data movement (ops.hip)
 void launch_rms_norm(hipStream_t s, const tdesc & src, const tdesc & dst, float eps, const tdesc * mul_w /* optional fused weight */);
+void launch_layer_norm(hipStream_t s, const tdesc & src, const tdesc & dst, float eps, const float * mul_w /* optional fused weight */, const tdesc * residual /* optional fused ADD */);
+void launch_argsort(hipStream_t s, const tdesc & src, const tdesc & dst, int descending);  // rows of f32 -> i32 permutation (stable)
+// element-wise forms outside ggml's unary enumeration, served by launch_unary: x^2 (SQR) and relu(x)^2 (RELU followed by SQR)
+#define MI_UNARY_SQR 1000
+#define MI_UNARY_RELU_SQR 1001
 void launch_binary(hipStream_t s, int op, const tdesc & a, const tdesc & b, const tdesc & dst);
 void launch_scale(hipStream_t s, const tdesc & src, const tdesc & dst, float scale, float bias);
 void launch_unary(hipStream_t s, int uop, const tdesc & src, const tdesc & dst);
@@ -359,6 +371,7 @@ void tu_touch_mmq_skinny(hipStream_t s);
 void tu_touch_mmq_q80(hipStream_t s);
 void tu_touch_ops(hipStream_t s);
 void tu_touch_fattn(hipStream_t s);
+void tu_touch_attn_f32(hipStream_t s);
 void tu_touch_fattn_mma(hipStream_t s);
 void tu_touch_tp_p2p(hipStream_t s);
 void tu_touch_kv_types(hipStream_t s);
@@ -377,6 +390,7 @@ inline void preload_kernel_files(hipStream_t s) {
     tu_touch_mmq_q80(s);
     tu_touch_ops(s);
     tu_touch_fattn(s);
+    tu_touch_attn_f32(s);
     tu_touch_fattn_mma(s);
     tu_touch_tp_p2p(s);
 }

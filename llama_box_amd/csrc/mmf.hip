@@ -13,8 +13,16 @@
 
 namespace mi355x {
 
-template <bool W16>
+// f32 -> bf16, nearest even (what ggml-cpu's from_float does to src1 when src0 is bf16), returned widened again
+__device__ __forceinline__ uint32_t mmf_bf16_bits(const float f) {
+    const uint32_t u = __float_as_uint(f);
+    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ float mmf_bf16_round(const float f) { return __uint_as_float(mmf_bf16_bits(f) << 16); }
+// WT: 0 = f32 src0 (true 32-bit products), 1 = f16, 2 = bf16 (src1 rounded to the same type first; f32 accumulation)
+template <int WT>
 __global__ void __launch_bounds__(256) k_mul_mat_f(const tdesc a, const tdesc b, const tdesc d, const int lpr, const int vec_ok) {
+    constexpr bool W16 = WT != 0;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int rpw = 64 / lpr;  // rows per wave
     const int sub = lane / lpr, sl = lane % lpr;
@@ -36,8 +44,8 @@ __global__ void __launch_bounds__(256) k_mul_mat_f(const tdesc a, const tdesc b,
                 const uint32_t u[4] = {t.x, t.y, t.z, t.w};
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    w[2 * i] = h2f((uint16_t) (u[i] & 0xFFFF));
-                    w[2 * i + 1] = h2f((uint16_t) (u[i] >> 16));
+                    w[2 * i] = WT == 2 ? __uint_as_float(u[i] << 16) : h2f((uint16_t) (u[i] & 0xFFFF));
+                    w[2 * i + 1] = WT == 2 ? __uint_as_float(u[i] & 0xFFFF0000u) : h2f((uint16_t) (u[i] >> 16));
                 }
             } else {
                 const float4 t0 = *(const float4 *) (wrow + k * 4), t1 = *(const float4 *) (wrow + k * 4 + 16);
@@ -47,15 +55,17 @@ __global__ void __launch_bounds__(256) k_mul_mat_f(const tdesc a, const tdesc b,
             float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const float xv = W16 ? h2f(f2h(x[i])) : x[i];
+                const float xv = WT == 2 ? mmf_bf16_round(x[i]) : (W16 ? h2f(f2h(x[i])) : x[i]);
                 acc = fmaf(w[i], xv, acc);
             }
         }
     } else {
         for (int64_t k = sl; k < K; k += lpr) {
-            const float wv = W16 ? h2f(*(const uint16_t *) (wrow + k * a.nb[0])) : *(const float *) (wrow + k * a.nb[0]);
+            const float wv = WT == 2 ? __uint_as_float((uint32_t) *(const uint16_t *) (wrow + k * a.nb[0]) << 16)
+                                     : (W16 ? h2f(*(const uint16_t *) (wrow + k * a.nb[0])) : *(const float *) (wrow + k * a.nb[0]));
             float xv = *(const float *) (xcol + k * b.nb[0]);
-            if (W16) xv = h2f(f2h(xv));
+            if (WT == 2) xv = mmf_bf16_round(xv);
+            else if (W16) xv = h2f(f2h(xv));
             acc = fmaf(wv, xv, acc);
         }
     }
@@ -73,6 +83,40 @@ __global__ void __launch_bounds__(256) k_mul_mat_f(const tdesc a, const tdesc b,
 // per MFMA —, which is still ~30x the dot kernel on these shapes.
 typedef _Float16 mmf_half8 __attribute__((ext_vector_type(8)));
 typedef float mmf_float16 __attribute__((ext_vector_type(16)));
+typedef float mmf_float4 __attribute__((ext_vector_type(4)));
+typedef __bf16 mmf_bf8 __attribute__((ext_vector_type(8)));
+// one MFMA step: eight f32 src1 values (x0, x1) rounded to src0's 16-bit type against eight src0 values (w); BF: both bf16 (v_mfma_*_bf16)
+template <bool BF> __device__ __forceinline__ mmf_float16 mmf_step32(const uint4 x0, const uint4 x1, const uint4 w, const mmf_float16 acc) {
+    if constexpr (BF) {
+        uint4 xb;
+        xb.x = mmf_bf16_bits(__uint_as_float(x0.x)) | (mmf_bf16_bits(__uint_as_float(x0.y)) << 16);
+        xb.y = mmf_bf16_bits(__uint_as_float(x0.z)) | (mmf_bf16_bits(__uint_as_float(x0.w)) << 16);
+        xb.z = mmf_bf16_bits(__uint_as_float(x1.x)) | (mmf_bf16_bits(__uint_as_float(x1.y)) << 16);
+        xb.w = mmf_bf16_bits(__uint_as_float(x1.z)) | (mmf_bf16_bits(__uint_as_float(x1.w)) << 16);
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(mmf_bf8, xb), __builtin_bit_cast(mmf_bf8, w), acc, 0, 0, 0);
+    } else {
+        const mmf_half8 x = {(_Float16) __builtin_bit_cast(float, x0.x), (_Float16) __builtin_bit_cast(float, x0.y), (_Float16) __builtin_bit_cast(float, x0.z),
+                             (_Float16) __builtin_bit_cast(float, x0.w), (_Float16) __builtin_bit_cast(float, x1.x), (_Float16) __builtin_bit_cast(float, x1.y),
+                             (_Float16) __builtin_bit_cast(float, x1.z), (_Float16) __builtin_bit_cast(float, x1.w)};
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(x, __builtin_bit_cast(mmf_half8, w), acc, 0, 0, 0);
+    }
+}
+template <bool BF> __device__ __forceinline__ mmf_float4 mmf_step16(const uint4 x0, const uint4 x1, const uint4 w, const mmf_float4 acc) {
+    if constexpr (BF) {
+        uint4 xb;
+        xb.x = mmf_bf16_bits(__uint_as_float(x0.x)) | (mmf_bf16_bits(__uint_as_float(x0.y)) << 16);
+        xb.y = mmf_bf16_bits(__uint_as_float(x0.z)) | (mmf_bf16_bits(__uint_as_float(x0.w)) << 16);
+        xb.z = mmf_bf16_bits(__uint_as_float(x1.x)) | (mmf_bf16_bits(__uint_as_float(x1.y)) << 16);
+        xb.w = mmf_bf16_bits(__uint_as_float(x1.z)) | (mmf_bf16_bits(__uint_as_float(x1.w)) << 16);
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mmf_bf8, xb), __builtin_bit_cast(mmf_bf8, w), acc, 0, 0, 0);
+    } else {
+        const mmf_half8 x = {(_Float16) __builtin_bit_cast(float, x0.x), (_Float16) __builtin_bit_cast(float, x0.y), (_Float16) __builtin_bit_cast(float, x0.z),
+                             (_Float16) __builtin_bit_cast(float, x0.w), (_Float16) __builtin_bit_cast(float, x1.x), (_Float16) __builtin_bit_cast(float, x1.y),
+                             (_Float16) __builtin_bit_cast(float, x1.z), (_Float16) __builtin_bit_cast(float, x1.w)};
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(x, __builtin_bit_cast(mmf_half8, w), acc, 0, 0, 0);
+    }
+}
+template <bool BF>
 __global__ void __launch_bounds__(256) k_mul_mat_f16_mma(const tdesc a, const tdesc b, const tdesc d) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r32 = lane & 31, g = lane >> 5;
@@ -102,12 +146,7 @@ __global__ void __launch_bounds__(256) k_mul_mat_f16_mma(const tdesc a, const td
             x1[u].x &= keep; x1[u].y &= keep; x1[u].z &= keep; x1[u].w &= keep;
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const mmf_half8 x = {(_Float16) __builtin_bit_cast(float, x0[u].x), (_Float16) __builtin_bit_cast(float, x0[u].y), (_Float16) __builtin_bit_cast(float, x0[u].z),
-                                 (_Float16) __builtin_bit_cast(float, x0[u].w), (_Float16) __builtin_bit_cast(float, x1[u].x), (_Float16) __builtin_bit_cast(float, x1[u].y),
-                                 (_Float16) __builtin_bit_cast(float, x1[u].z), (_Float16) __builtin_bit_cast(float, x1[u].w)};
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(x, __builtin_bit_cast(mmf_half8, w[u]), acc, 0, 0, 0);
-        }
+        for (int u = 0; u < 4; ++u) acc = mmf_step32<BF>(x0[u], x1[u], w[u], acc);
     }
     // lane: src0 row row0 + r32; register i: src1 column col0 + (i & 3) + 8 (i >> 2) + 4 g
     const int64_t row = row0 + r32;
@@ -199,8 +238,7 @@ template <int GH> static void launch_xres_t(hipStream_t s, const tdesc & a, cons
 // over thousands of cells — 128 waves of the kernel above, each walking all of K, took 170 us), and for 2..15 columns: 16 x 16 tiles
 // on v_mfma_f32_16x16x32_f16 (A: src1 column m = lane & 15, B: src0 row n = lane & 15, k-group lane >> 4), the NWK waves of a
 // workgroup take the K steps of ONE tile in turn and add up through LDS in wave order (deterministic).
-typedef float mmf_float4 __attribute__((ext_vector_type(4)));
-template <int NWK>
+template <int NWK, bool BF>
 __global__ void __launch_bounds__(64 * NWK) k_mul_mat_f16_mma16(const tdesc a, const tdesc b, const tdesc d) {
     __shared__ mmf_float4 red[NWK][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -228,12 +266,7 @@ __global__ void __launch_bounds__(64 * NWK) k_mul_mat_f16_mma16(const tdesc a, c
             x1[u].x &= keep; x1[u].y &= keep; x1[u].z &= keep; x1[u].w &= keep;
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const mmf_half8 x = {(_Float16) __builtin_bit_cast(float, x0[u].x), (_Float16) __builtin_bit_cast(float, x0[u].y), (_Float16) __builtin_bit_cast(float, x0[u].z),
-                                 (_Float16) __builtin_bit_cast(float, x0[u].w), (_Float16) __builtin_bit_cast(float, x1[u].x), (_Float16) __builtin_bit_cast(float, x1[u].y),
-                                 (_Float16) __builtin_bit_cast(float, x1[u].z), (_Float16) __builtin_bit_cast(float, x1[u].w)};
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(x, __builtin_bit_cast(mmf_half8, w[u]), acc, 0, 0, 0);
-        }
+        for (int u = 0; u < 4; ++u) acc = mmf_step16<BF>(x0[u], x1[u], w[u], acc);
     }
     red[wave][lane] = acc;
     __syncthreads();
@@ -694,12 +727,14 @@ template <int G> static void launch_gqa_t(hipStream_t s, const tdesc & a, const 
 
 void launch_mul_mat_f(hipStream_t s, const tdesc & a, const tdesc & b, const tdesc & d, float * ws, size_t ws_bytes) {
     const int64_t K = a.ne[0];
-    const bool w16 = a.type == GGML_TYPE_F16;
+    const bool bf = a.type == GGML_TYPE_BF16;           // bf16 src0: the same tilings on the bf16 matrix-core instructions
+    const bool w16 = a.type == GGML_TYPE_F16 || bf;     // a 2-byte src0
     const int esz = w16 ? 2 : 4;
+    if (a.ne[1] == 0 || b.ne[1] * b.ne[2] * b.ne[3] == 0) return;
     // 16-byte vector path: contiguous dim 0 on both sides, K multiple of 8, every row start 16-byte aligned
     bool vec_ok = a.nb[0] == esz && b.nb[0] == 4 && (K % 8) == 0 && (((uintptr_t) a.data) & 15) == 0 && (((uintptr_t) b.data) & 15) == 0;
     for (int i = 1; i < 4; ++i) vec_ok = vec_ok && (a.nb[i] % 16) == 0 && (b.nb[i] % 16) == 0;
-    if (w16 && vec_ok && ws && d.nb[0] == 4 && d.nb[1] == d.ne[0] * 4 && d.nb[2] == d.nb[1] * d.ne[1] && d.nb[3] == d.nb[2] * d.ne[2]) {
+    if (w16 && !bf && vec_ok && ws && d.nb[0] == 4 && d.nb[1] == d.ne[0] * 4 && d.nb[2] == d.nb[1] * d.ne[1] && d.nb[3] == d.nb[2] * d.ne[2]) {
         int64_t Kc = 0;
         const int ks = mmf_ksplit_slices(a, b, &Kc);
         if (ks > 1 && mul_mat_f_workspace_bytes(a, b) <= ws_bytes) {
@@ -715,12 +750,15 @@ void launch_mul_mat_f(hipStream_t s, const tdesc & a, const tdesc & b, const tde
         const int64_t waves32 = ((a.ne[1] + 31) / 32) * ((b.ne[1] + 31) / 32) * b.ne[2] * b.ne[3];
         if (b.ne[1] < 16 || (K >= 1024 && waves32 < 2048)) {  // few tiles, long rows (or a handful of columns): split K inside the workgroup
             dim3 grid((unsigned) ((a.ne[1] + 15) / 16), (unsigned) ((b.ne[1] + 15) / 16), (unsigned) (b.ne[2] * b.ne[3]));
-            if (K >= 4096) hipLaunchKernelGGL(k_mul_mat_f16_mma16<16>, grid, dim3(1024), 0, s, a, b, d);
-            else hipLaunchKernelGGL(k_mul_mat_f16_mma16<8>, grid, dim3(512), 0, s, a, b, d);
+            if (bf) {
+                if (K >= 4096) hipLaunchKernelGGL((k_mul_mat_f16_mma16<16, true>), grid, dim3(1024), 0, s, a, b, d);
+                else hipLaunchKernelGGL((k_mul_mat_f16_mma16<8, true>), grid, dim3(512), 0, s, a, b, d);
+            } else if (K >= 4096) hipLaunchKernelGGL((k_mul_mat_f16_mma16<16, false>), grid, dim3(1024), 0, s, a, b, d);
+            else hipLaunchKernelGGL((k_mul_mat_f16_mma16<8, false>), grid, dim3(512), 0, s, a, b, d);
             return;
         }
     }
-    if (w16 && vec_ok && b.ne[1] >= 16 && K <= 128 && a.ne[1] >= 256 && b.ne[2] % a.ne[2] == 0) {  // short rows, many of them (K.Q): columns resident
+    if (w16 && !bf && vec_ok && b.ne[1] >= 16 && K <= 128 && a.ne[1] >= 256 && b.ne[2] % a.ne[2] == 0) {  // short rows, many of them (K.Q): columns resident
         const int64_t gq = b.ne[2] / a.ne[2];
         if (gq % 2 == 0) launch_xres_t<2>(s, a, b, d);  // (4 heads' columns = 128 registers: with the row buffers past 256, one wave per SIMD, or spills)
         else launch_xres_t<1>(s, a, b, d);
@@ -728,10 +766,11 @@ void launch_mul_mat_f(hipStream_t s, const tdesc & a, const tdesc & b, const tde
     }
     if (w16 && vec_ok && b.ne[1] >= 16) {  // a batch of columns: the matrix cores
         dim3 grid((unsigned) ((a.ne[1] + 63) / 64), (unsigned) ((b.ne[1] + 63) / 64), (unsigned) (b.ne[2] * b.ne[3]));
-        hipLaunchKernelGGL(k_mul_mat_f16_mma, grid, dim3(256), 0, s, a, b, d);
+        if (bf) hipLaunchKernelGGL(k_mul_mat_f16_mma<true>, grid, dim3(256), 0, s, a, b, d);
+        else hipLaunchKernelGGL(k_mul_mat_f16_mma<false>, grid, dim3(256), 0, s, a, b, d);
         return;
     }
-    if (w16 && vec_ok && b.ne[1] == 1 && a.ne[3] == 1 && b.ne[3] == 1 && b.ne[2] % a.ne[2] == 0 && a.ne[1] >= 64) {  // a decode step's K.q / V^T.p
+    if (w16 && !bf && vec_ok && b.ne[1] == 1 && a.ne[3] == 1 && b.ne[3] == 1 && b.ne[2] % a.ne[2] == 0 && a.ne[1] >= 64) {  // a decode step's K.q / V^T.p
         switch (b.ne[2] / a.ne[2]) {
             case 1: launch_gqa_t<1>(s, a, b, d); return;
             case 2: launch_gqa_t<2>(s, a, b, d); return;
@@ -752,8 +791,150 @@ void launch_mul_mat_f(hipStream_t s, const tdesc & a, const tdesc & b, const tde
     }
     const int rows_per_block = 4 * (64 / lpr);
     dim3 grid((unsigned) ((a.ne[1] + rows_per_block - 1) / rows_per_block), (unsigned) b.ne[1], (unsigned) (b.ne[2] * b.ne[3]));
-    if (w16) hipLaunchKernelGGL(k_mul_mat_f<true>, grid, dim3(256), 0, s, a, b, d, lpr, vec_ok ? 1 : 0);
-    else hipLaunchKernelGGL(k_mul_mat_f<false>, grid, dim3(256), 0, s, a, b, d, lpr, vec_ok ? 1 : 0);
+    if (bf) hipLaunchKernelGGL(k_mul_mat_f<2>, grid, dim3(256), 0, s, a, b, d, lpr, vec_ok ? 1 : 0);
+    else if (w16) hipLaunchKernelGGL(k_mul_mat_f<1>, grid, dim3(256), 0, s, a, b, d, lpr, vec_ok ? 1 : 0);
+    else hipLaunchKernelGGL(k_mul_mat_f<0>, grid, dim3(256), 0, s, a, b, d, lpr, vec_ok ? 1 : 0);
+}
+
+// ------------------------------------------------------------------------------------------------ MUL_MAT_ID (mixture of experts)
+// as: [K, N, n_expert] f32 / f16 / bf16; b: [K, n_b, T] f32 (n_b = 1: every used expert reads the token's one activation row, or n_b = n_used);
+// ids: [n_used, T] i32; d: [N, n_used, T] f32.  Column (u, t) is as[ids[u, t]] . b[:, u % n_b, t], with k_mul_mat_f's arithmetic
+// (src1 rounded to src0's 16-bit type, f32 accumulation).
+//   k_mul_mat_id      — one (u, t) column per workgroup row: a decode step or a few tokens; the expert's rows stream once per column.
+//   k_mul_mat_id_mma  — batches: the (u, t) columns are first grouped by expert (k_moe_group: counts, offsets and the column list, one
+//                       workgroup), then every expert's matrix is multiplied with ITS columns on the matrix cores — 32 x 32 tiles as in
+//                       k_mul_mat_f16_mma, the columns gathered through the list, the results scattered to their (u, t) places.
+template <int WT>
+__global__ void __launch_bounds__(256) k_mul_mat_id(const tdesc a, const tdesc b, const tdesc ids, const tdesc d, const int lpr) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int rpw = 64 / lpr;
+    const int sub = lane / lpr, sl = lane % lpr;
+    const int64_t i01 = ((int64_t) blockIdx.x * 4 + wave) * rpw + sub;
+    const int64_t u = blockIdx.y, t = blockIdx.z;
+    const int32_t e = *(const int32_t *) (ids.data + u * ids.nb[0] + t * ids.nb[1]);
+    if (e < 0 || e >= a.ne[2]) return;  // (an index outside the experts: the column is left as it is)
+    const int64_t K = a.ne[0];
+    const bool live = i01 < a.ne[1];
+    const int64_t r = live ? i01 : a.ne[1] - 1;
+    const char * wrow = a.data + r * a.nb[1] + (int64_t) e * a.nb[2];
+    const char * xcol = b.data + (u % b.ne[1]) * b.nb[1] + t * b.nb[2];
+    float acc = 0.0f;
+    for (int64_t k = sl; k < K; k += lpr) {
+        float wv, xv = *(const float *) (xcol + k * b.nb[0]);
+        if (WT == 2) { wv = __uint_as_float((uint32_t) *(const uint16_t *) (wrow + k * 2) << 16); xv = mmf_bf16_round(xv); }
+        else if (WT == 1) { wv = h2f(*(const uint16_t *) (wrow + k * 2)); xv = h2f(f2h(xv)); }
+        else wv = *(const float *) (wrow + k * 4);
+        acc = fmaf(wv, xv, acc);
+    }
+    for (int o = lpr >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+    if (live && sl == 0) *(float *) (d.data + i01 * d.nb[0] + u * d.nb[1] + t * d.nb[2]) = acc;
+}
+
+// columns grouped by expert: cnt[e], off[e] (exclusive prefix) and list[off[e] + i] = u + n_used * t, in (t, u) order within an expert
+__global__ void __launch_bounds__(256) k_moe_group(const tdesc ids, const int n_expert, int32_t * __restrict__ cnt, int32_t * __restrict__ off, int32_t * __restrict__ list) {
+    __shared__ int32_t s_cnt[256], s_off[256];
+    const int64_t n_used = ids.ne[0], T = ids.ne[1], n = n_used * T;
+    // (thread e owns expert e: a scan of all columns per thread — a few thousand index reads from L2, no atomics, a deterministic order)
+    for (int e0 = 0; e0 < n_expert; e0 += 256) {
+        const int e = e0 + threadIdx.x;
+        int c = 0;
+        if (e < n_expert)
+            for (int64_t i = 0; i < n; ++i) c += *(const int32_t *) (ids.data + (i % n_used) * ids.nb[0] + (i / n_used) * ids.nb[1]) == e ? 1 : 0;
+        s_cnt[threadIdx.x] = c;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            int base = e0 == 0 ? 0 : off[e0 - 1] + cnt[e0 - 1];
+            for (int x = 0; x < 256 && e0 + x < n_expert; ++x) { s_off[x] = base; base += s_cnt[x]; }
+        }
+        __syncthreads();
+        if (e < n_expert) {
+            cnt[e] = c;
+            off[e] = s_off[threadIdx.x];
+            int at = s_off[threadIdx.x];
+            for (int64_t i = 0; i < n; ++i)
+                if (*(const int32_t *) (ids.data + (i % n_used) * ids.nb[0] + (i / n_used) * ids.nb[1]) == e) list[at++] = (int32_t) i;
+        }
+        __syncthreads();
+    }
+}
+
+template <bool BF>
+__global__ void __launch_bounds__(256) k_mul_mat_id_mma(const tdesc a, const tdesc b, const tdesc d, const int64_t n_used, const int32_t * __restrict__ cnt, const int32_t * __restrict__ off,
+                                                        const int32_t * __restrict__ list) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r32 = lane & 31, g = lane >> 5;
+    const int e = blockIdx.z;
+    const int n_cols = cnt[e];
+    const int64_t row0 = ((int64_t) blockIdx.x * 2 + (wave & 1)) * 32;
+    if (row0 >= a.ne[1]) return;
+    const int32_t * cols = list + off[e];
+    const int64_t K = a.ne[0];
+    const char * wrow = a.data + std::min<int64_t>(row0 + r32, a.ne[1] - 1) * a.nb[1] + (int64_t) e * a.nb[2] + g * 16;
+    // a workgroup walks the expert's column tiles (grid.y strides them): experts with many columns are shared out, those with few end at once
+    for (int64_t col0 = ((int64_t) blockIdx.y * 2 + (wave >> 1)) * 32; col0 < n_cols; col0 += (int64_t) gridDim.y * 64) {
+        const int32_t ci = cols[std::min<int64_t>(col0 + r32, n_cols - 1)];
+        const int64_t cu = ci % n_used, ct = ci / n_used;
+        const char * xcol = b.data + (cu % b.ne[1]) * b.nb[1] + ct * b.nb[2] + g * 32;
+        mmf_float16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        for (int64_t k = 0; k < K; k += 64) {
+            uint4 w[4], x0[4], x1[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int64_t kk = k + 16 * u;
+                const bool in = kk + 8 * g < K;
+                const int64_t kc = in ? kk : -8 * g;
+                const uint32_t keep = in ? 0xFFFFFFFFu : 0u;
+                w[u] = *(const uint4 *) (wrow + kc * 2);
+                x0[u] = *(const uint4 *) (xcol + kc * 4);
+                x1[u] = *(const uint4 *) (xcol + kc * 4 + 16);
+                w[u].x &= keep; w[u].y &= keep; w[u].z &= keep; w[u].w &= keep;
+                x0[u].x &= keep; x0[u].y &= keep; x0[u].z &= keep; x0[u].w &= keep;
+                x1[u].x &= keep; x1[u].y &= keep; x1[u].z &= keep; x1[u].w &= keep;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) acc = mmf_step32<BF>(x0[u], x1[u], w[u], acc);
+        }
+        const int64_t row = row0 + r32;
+        if (row < a.ne[1]) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int64_t c = col0 + (i & 3) + 8 * (i >> 2) + 4 * g;
+                if (c < n_cols) {
+                    const int32_t oi = cols[c];
+                    *(float *) (d.data + row * d.nb[0] + (oi % n_used) * d.nb[1] + (oi / n_used) * d.nb[2]) = acc[i];
+                }
+            }
+        }
+    }
+}
+
+size_t mul_mat_id_workspace_bytes(const tdesc & as, const tdesc & ids) {
+    return ((size_t) as.ne[2] * 2 + (size_t) (ids.ne[0] * ids.ne[1])) * sizeof(int32_t) + 256;
+}
+// grouped: the column lists made by an earlier call over the same ids (the down projection follows the up projection) are used again
+void launch_mul_mat_id(hipStream_t s, const tdesc & as, const tdesc & b, const tdesc & ids, const tdesc & d, void * ws, size_t ws_bytes, bool lists_valid) {
+    const int64_t K = as.ne[0], n_used = ids.ne[0], T = ids.ne[1];
+    if (as.ne[1] == 0 || n_used * T == 0) return;
+    const bool bf = as.type == GGML_TYPE_BF16, w16 = bf || as.type == GGML_TYPE_F16;
+    bool vec_ok = w16 && as.nb[0] == 2 && b.nb[0] == 4 && (K % 8) == 0 && (((uintptr_t) as.data) & 15) == 0 && (((uintptr_t) b.data) & 15) == 0;
+    for (int i = 1; i < 3; ++i) vec_ok = vec_ok && (as.nb[i] % 16) == 0 && (b.nb[i] % 16) == 0;
+    if (vec_ok && n_used * T >= 64 && as.ne[2] <= 65535 && ws && mul_mat_id_workspace_bytes(as, ids) <= ws_bytes) {
+        int32_t * cnt = (int32_t *) ws, * off = cnt + as.ne[2], * list = off + as.ne[2];
+        if (!lists_valid) hipLaunchKernelGGL(k_moe_group, dim3(1), dim3(256), 0, s, ids, (int) as.ne[2], cnt, off, list);
+        // column tiles per expert in the grid: enough for an even spread (the loop inside covers an expert that drew more)
+        const int64_t even = (n_used * T + as.ne[2] - 1) / as.ne[2];
+        const dim3 grid((unsigned) ((as.ne[1] + 63) / 64), (unsigned) std::max<int64_t>(1, std::min<int64_t>(64, (even + 63) / 64 * 2)), (unsigned) as.ne[2]);
+        if (bf) hipLaunchKernelGGL(k_mul_mat_id_mma<true>, grid, dim3(256), 0, s, as, b, d, n_used, cnt, off, list);
+        else hipLaunchKernelGGL(k_mul_mat_id_mma<false>, grid, dim3(256), 0, s, as, b, d, n_used, cnt, off, list);
+        return;
+    }
+    int lpr = 64;
+    while (lpr > 8 && (int64_t) (lpr / 2) >= K) lpr >>= 1;
+    const int rows_per_block = 4 * (64 / lpr);
+    const dim3 grid((unsigned) ((as.ne[1] + rows_per_block - 1) / rows_per_block), (unsigned) n_used, (unsigned) T);
+    if (bf) hipLaunchKernelGGL(k_mul_mat_id<2>, grid, dim3(256), 0, s, as, b, ids, d, lpr);
+    else if (w16) hipLaunchKernelGGL(k_mul_mat_id<1>, grid, dim3(256), 0, s, as, b, ids, d, lpr);
+    else hipLaunchKernelGGL(k_mul_mat_id<0>, grid, dim3(256), 0, s, as, b, ids, d, lpr);
 }
 
 MI_TU_TOUCH(mmf)

@@ -8,6 +8,7 @@
 
 #include "dev_util.h"
 #include "kernels.h"
+#include "kv_quant.h"
 
 namespace mi355x {
 
@@ -132,6 +133,69 @@ void launch_rms_norm_mul_q80_panel(hipStream_t s, const tdesc & src, float eps, 
     hipLaunchKernelGGL(k_rms_norm<true>, dim3((unsigned) rows), dim3(256), 0, s, src, src, eps, w, (char *) q80_panel);
 }
 
+// ------------------------------------------------------------------------------------------------ NORM (layer normalisation)
+// y = (x - mean) / sqrt(var + eps) [* w] [+ r], var = mean of the squared deviations (two passes over a row kept in registers / L2; sums in f64
+// like RMS_NORM's).  w: optional weight of the MUL that follows; r: optional residual rows of the ADD behind that (same shape as the output).
+__global__ void __launch_bounds__(256) k_layer_norm(const tdesc a, const tdesc d, const float eps, const float * __restrict__ w, const tdesc r, const int has_r) {
+    __shared__ double sh[4];
+    const int64_t row = blockIdx.x;
+    const int64_t i1 = row % a.ne[1], i2 = (row / a.ne[1]) % a.ne[2], i3 = row / (a.ne[1] * a.ne[2]);
+    const float * __restrict__ x = (const float *) (a.data + i1 * a.nb[1] + i2 * a.nb[2] + i3 * a.nb[3]);
+    float * __restrict__ y = (float *) (d.data + i1 * d.nb[1] + i2 * d.nb[2] + i3 * d.nb[3]);
+    const float * __restrict__ rr = has_r ? (const float *) (r.data + i1 * r.nb[1] + i2 * r.nb[2] + i3 * r.nb[3]) : nullptr;
+    const int64_t n = a.ne[0];
+    double s = 0.0;
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) s += (double) x[i];
+    s = block_sum_d(s, sh);
+    const float mean = (float) (s / (double) n);
+    __syncthreads();
+    double q = 0.0;
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+        const float dv = x[i] - mean;
+        q += (double) (dv * dv);
+    }
+    q = block_sum_d(q, sh);
+    const float var = (float) (q / (double) n);
+    const float scale = 1.0f / sqrtf(var + eps);
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+        float v = (x[i] - mean) * scale;
+        if (w) v *= w[i];
+        if (rr) v += rr[i];
+        y[i] = v;
+    }
+}
+void launch_layer_norm(hipStream_t s, const tdesc & src, const tdesc & dst, float eps, const float * mul_w, const tdesc * residual) {
+    const int64_t rows = src.ne[1] * src.ne[2] * src.ne[3];
+    if (rows == 0) return;
+    hipLaunchKernelGGL(k_layer_norm, dim3((unsigned) rows), dim3(256), 0, s, src, dst, eps, mul_w, residual ? *residual : src, residual ? 1 : 0);
+}
+
+// ------------------------------------------------------------------------------------------------ ARGSORT
+// one workgroup per row: element i's place is the number of elements that sort before it (ties keep their index order), so the result is the
+// stable sort's permutation; rows of up to a few thousand entries (router logits)
+__global__ void __launch_bounds__(256) k_argsort(const tdesc a, const tdesc d, const int descending) {
+    const int64_t row = blockIdx.x;
+    const int64_t i1 = row % a.ne[1], i2 = (row / a.ne[1]) % a.ne[2], i3 = row / (a.ne[1] * a.ne[2]);
+    const float * __restrict__ x = (const float *) (a.data + i1 * a.nb[1] + i2 * a.nb[2] + i3 * a.nb[3]);
+    int32_t * __restrict__ y = (int32_t *) (d.data + i1 * d.nb[1] + i2 * d.nb[2] + i3 * d.nb[3]);
+    const int n = (int) a.ne[0];
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const float v = x[i];
+        int before = 0;
+        for (int j = 0; j < n; ++j) {
+            const float u = x[j];
+            const bool first = descending ? (u > v) : (u < v);
+            before += (first || (u == v && j < i)) ? 1 : 0;
+        }
+        y[before] = i;
+    }
+}
+void launch_argsort(hipStream_t s, const tdesc & src, const tdesc & dst, int descending) {
+    const int64_t rows = src.ne[1] * src.ne[2] * src.ne[3];
+    if (rows == 0) return;
+    hipLaunchKernelGGL(k_argsort, dim3((unsigned) rows), dim3(256), 0, s, src, dst, descending);
+}
+
 // ------------------------------------------------------------------------------------------------ ADD/SUB/MUL/DIV
 __global__ void __launch_bounds__(256) k_binary(const int op, const tdesc a, const tdesc b, const tdesc d) {
     const int64_t row = blockIdx.x;
@@ -196,6 +260,10 @@ __global__ void __launch_bounds__(256) k_unary(const int uop, const float * __re
             case GGML_UNARY_OP_NEG: r = -v; break;
             case GGML_UNARY_OP_EXP: r = expf(v); break;
             case GGML_UNARY_OP_TANH: r = tanhf(v); break;
+            case GGML_UNARY_OP_GELU_ERF: r = 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f)); break;
+            case GGML_UNARY_OP_GELU: r = 0.5f * v * (1.0f + tanhf(0.79788456080286535588f * (v + 0.044715f * v * v * v))); break;
+            case MI_UNARY_SQR: r = v * v; break;
+            case MI_UNARY_RELU_SQR: r = v > 0.f ? v * v : 0.f; break;
             default: r = 1.f / (1.f + expf(-v)); break;  // SIGMOID
         }
         y[i] = r;
@@ -307,6 +375,7 @@ __device__ __forceinline__ float dequant_elem(const int type, const uint8_t * __
     switch (type) {
         case GGML_TYPE_F32: return ((const float *) row)[i];
         case GGML_TYPE_F16: return h2f(((const uint16_t *) row)[i]);
+        case GGML_TYPE_BF16: return __uint_as_float((uint32_t) ((const uint16_t *) row)[i] << 16);
         case GGML_TYPE_Q8_0: {
             const uint8_t * b = row + (i >> 5) * 34;
             return (float) (int8_t) b[2 + (i & 31)] * h2f(ld16(b));
@@ -374,7 +443,7 @@ __global__ void __launch_bounds__(256) k_set_rows(const tdesc a, const tdesc idx
     const int64_t i1 = *(const int64_t *) (idx.data + i01 * idx.nb[0] + (i02 % idx.ne[1]) * idx.nb[1] + (i03 % idx.ne[2]) * idx.nb[2]);
     const float * __restrict__ x = (const float *) (a.data + i01 * a.nb[1] + i02 * a.nb[2] + i03 * a.nb[3]);
     char * __restrict__ p = d.data + i1 * d.nb[1] + i02 * d.nb[2] + i03 * d.nb[3];
-    if ((nc & 3) == 0 && ((((uintptr_t) x) | ((uintptr_t) p)) & 15) == 0) {
+    if (d.type != GGML_TYPE_BF16 && (nc & 3) == 0 && ((((uintptr_t) x) | ((uintptr_t) p)) & 15) == 0) {
         const int64_t n4 = nc >> 2;
         for (int64_t i0 = threadIdx.x; i0 < n4; i0 += 1024) {
             float4 v[4];
@@ -398,6 +467,7 @@ __global__ void __launch_bounds__(256) k_set_rows(const tdesc a, const tdesc idx
         return;
     }
     if (d.type == GGML_TYPE_F16) for (int64_t i = threadIdx.x; i < nc; i += blockDim.x) ((uint16_t *) p)[i] = f2h(x[i]);
+    else if (d.type == GGML_TYPE_BF16) for (int64_t i = threadIdx.x; i < nc; i += blockDim.x) ((uint16_t *) p)[i] = f2bf(x[i]);
     else for (int64_t i = threadIdx.x; i < nc; i += blockDim.x) ((float *) p)[i] = x[i];
 }
 void launch_set_rows(hipStream_t s, const tdesc & a, const tdesc & idx, const tdesc & d) {

@@ -346,6 +346,48 @@ struct ggml_tensor * ggml_rms_norm(struct ggml_context * ctx, struct ggml_tensor
     return r;
 }
 
+// layer normalisation without affine terms: (x - mean) / sqrt(var + eps) over dim 0
+struct ggml_tensor * ggml_norm(struct ggml_context * ctx, struct ggml_tensor * a, float eps) {
+    ggml_tensor * r = dup_tensor(ctx, a);
+    set_f32(r, 0, eps);
+    r->op = GGML_OP_NORM;
+    r->src[0] = a;
+    return r;
+}
+struct ggml_tensor * ggml_sqr(struct ggml_context * ctx, struct ggml_tensor * a) {
+    ggml_tensor * r = dup_tensor(ctx, a);
+    r->op = GGML_OP_SQR;
+    r->src[0] = a;
+    return r;
+}
+// indices that sort every row of a (dim 0); order: 0 ascending, 1 descending
+struct ggml_tensor * ggml_argsort(struct ggml_context * ctx, struct ggml_tensor * a, int order) {
+    LITE_ASSERT(a->type == GGML_TYPE_F32);
+    ggml_tensor * r = ggml_new_tensor(ctx, GGML_TYPE_I32, GGML_MAX_DIMS, a->ne);
+    r->op_params[0] = order;
+    r->op = GGML_OP_ARGSORT;
+    r->src[0] = a;
+    return r;
+}
+// the k largest entries of every row: a view of the first k columns of the descending argsort (as ggml_top_k)
+struct ggml_tensor * ggml_top_k(struct ggml_context * ctx, struct ggml_tensor * a, int k) {
+    LITE_ASSERT(a->ne[0] >= k);
+    ggml_tensor * s = ggml_argsort(ctx, a, 1);
+    return ggml_view_4d(ctx, s, k, s->ne[1], s->ne[2], s->ne[3], s->nb[1], s->nb[2], s->nb[3], 0);
+}
+// as: [K, N, n_expert]; b: [K, n_used or 1, T]; ids: [n_used, T] i32 -> [N, n_used, T]: column (u, t) is as[ids[u, t]] . b[:, u or 0, t]
+struct ggml_tensor * ggml_mul_mat_id(struct ggml_context * ctx, struct ggml_tensor * as, struct ggml_tensor * b, struct ggml_tensor * ids) {
+    LITE_ASSERT(as->ne[3] == 1 && b->ne[3] == 1 && ids->ne[2] == 1 && ids->ne[3] == 1 && ids->type == GGML_TYPE_I32);
+    LITE_ASSERT(ids->ne[1] == b->ne[2] && as->ne[0] == b->ne[0] && ids->ne[0] % b->ne[1] == 0);
+    const int64_t ne[4] = {as->ne[1], ids->ne[0], b->ne[2], 1};
+    ggml_tensor * r = ggml_new_tensor(ctx, GGML_TYPE_F32, 4, ne);
+    r->op = GGML_OP_MUL_MAT_ID;
+    r->src[0] = as;
+    r->src[1] = b;
+    r->src[2] = ids;
+    return r;
+}
+
 struct ggml_tensor * ggml_mul_mat(struct ggml_context * ctx, struct ggml_tensor * a, struct ggml_tensor * b) {
     LITE_ASSERT(a->ne[0] == b->ne[0] && b->ne[2] % a->ne[2] == 0 && b->ne[3] % a->ne[3] == 0);
     LITE_ASSERT(a->nb[0] <= a->nb[1]);  // !ggml_is_transposed(a)

@@ -78,6 +78,11 @@ struct ggml_tensor * ggml_div(struct ggml_context * ctx, struct ggml_tensor * a,
 struct ggml_tensor * ggml_scale(struct ggml_context * ctx, struct ggml_tensor * a, float s);
 struct ggml_tensor * ggml_scale_bias(struct ggml_context * ctx, struct ggml_tensor * a, float s, float b);
 struct ggml_tensor * ggml_rms_norm(struct ggml_context * ctx, struct ggml_tensor * a, float eps);
+struct ggml_tensor * ggml_norm(struct ggml_context * ctx, struct ggml_tensor * a, float eps);
+struct ggml_tensor * ggml_sqr(struct ggml_context * ctx, struct ggml_tensor * a);
+struct ggml_tensor * ggml_argsort(struct ggml_context * ctx, struct ggml_tensor * a, int order);
+struct ggml_tensor * ggml_top_k(struct ggml_context * ctx, struct ggml_tensor * a, int k);
+struct ggml_tensor * ggml_mul_mat_id(struct ggml_context * ctx, struct ggml_tensor * as, struct ggml_tensor * b, struct ggml_tensor * ids);
 struct ggml_tensor * ggml_mul_mat(struct ggml_context * ctx, struct ggml_tensor * a, struct ggml_tensor * b);
 void ggml_mul_mat_set_prec(struct ggml_tensor * a, enum ggml_prec prec);
 struct ggml_tensor * ggml_get_rows(struct ggml_context * ctx, struct ggml_tensor * a, struct ggml_tensor * b);

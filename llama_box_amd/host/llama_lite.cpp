@@ -14,6 +14,8 @@
 #include <vector>
 
 #include "gguf_lite.h"
+#include "json_lite.h"
+#include "safetensors_lite.h"
 
 #define LLM_ASSERT(x)                                                                           \
     do {                                                                                        \
@@ -326,6 +328,24 @@ struct llm_layer {
     ggml_tensor *attn_norm = nullptr, *wq = nullptr, *wk = nullptr, *wv = nullptr, *wo = nullptr;
     ggml_tensor *bq = nullptr, *bk = nullptr, *bv = nullptr;
     ggml_tensor *ffn_norm = nullptr, *ffn_gate = nullptr, *ffn_up = nullptr, *ffn_down = nullptr;
+    // models described layer by layer (llm_layer_cfg): norms behind the sublayers, the attention output gate, the experts and their router
+    ggml_tensor *attn_post_norm = nullptr, *ffn_post_norm = nullptr, *attn_gate = nullptr;
+    ggml_tensor *ffn_gate_inp = nullptr, *ffn_up_exps = nullptr, *ffn_down_exps = nullptr;
+};
+
+// one layer of a model whose config lists its layers one by one (sizes and constants may differ from layer to layer)
+enum llm_mlp_kind { LLM_MLP_NONE = 0, LLM_MLP_DENSE = 1, LLM_MLP_MOE = 2 };
+struct llm_layer_cfg {
+    int n_head = 0, n_head_kv = 0, dk = 0, dv = 0;  // query heads, key/value heads, per-head query/key size, per-head value size
+    int rot_dims = 0;                               // leading dims of every head that are rotated, as neighbouring pairs
+    float rot_base = 10000.0f, scale = 1.0f;
+    int chunk = 0;                                  // > 0: a position sees only earlier positions with the same floor(pos / chunk)
+    bool sink = false;                              // soft-max denominator carries one more term exp(0): a sink without a value
+    bool v_mix = false;                             // values are blended with those of the first such layer ...
+    float v_lambda = 0.0f;                          // ... v <- (1 - lambda) v + lambda v_first
+    bool out_gate = false;                          // heads are multiplied by sigmoid(W_g h) before the output projection
+    int mlp = LLM_MLP_NONE, n_ff = 0, n_expert = 0, n_top = 0;
+    int mask_id = 0;                                // index into llm_model::mask_chunks
 };
 
 struct tensor_plan {
@@ -355,6 +375,13 @@ struct llm_model {
     uint64_t stream_bytes = 0, total_bytes = 0;
     int n_dev = 1;               // -sm layer: devices the layers are spread over (llm_model_synth_layer_split)
     std::vector<int> layer_dev;  // ... and which of them holds layer il
+    // per-layer description (empty for the uniform llama / qwen2 classes)
+    std::vector<llm_layer_cfg> lcfg;
+    std::vector<int> mask_chunks;        // the distinct chunk sizes of the layers (0 = plain causal): one attention mask each
+    float embd_scale = 1.0f;
+    ggml_tensor * attn_sinks = nullptr;  // zeros, one per query head: the sink's score
+    ggml_type wtype = GGML_TYPE_F32;     // type of the matrices (and the default type of the cache)
+    int max_embd_k = 0, max_embd_v = 0;  // widest K / V cache row over the layers
 };
 
 static bool use_more_bits(int i, int n) { return i < n / 8 || i >= 7 * n / 8 || (i - n / 8) % 3 == 2; }
@@ -695,6 +722,290 @@ extern "C" struct llm_model * llm_model_load(const char * path, ggml_backend_buf
     return m;
 }
 
+// ---------------------------------------------------------------------------------------------- models from a checkpoint folder
+// config.json names the architecture and lists the layers; model.safetensors holds bf16 matrices stored [out, in].  The tensors are
+// re-named to the framework's own scheme (token_embd, blk.N.attn_q, ...); the experts of a layer are stacked into one 3-d tensor per
+// projection, the form MUL_MAT_ID reads.
+static float bf16_to_f32(uint16_t h) {
+    const uint32_t x = (uint32_t) h << 16;
+    float f;
+    memcpy(&f, &x, 4);
+    return f;
+}
+static uint16_t f32_to_bf16(float f) {  // round to nearest even
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t) ((x >> 16) | 0x40);
+    return (uint16_t) ((x + 0x7FFFu + ((x >> 16) & 1u)) >> 16);
+}
+
+struct dir_tensor {               // one framework tensor and where its values come from
+    std::string name;             // framework name
+    ggml_type type;
+    int64_t ne[3];
+    std::vector<std::string> src; // checkpoint tensors, stacked along the last dim (one entry unless experts)
+    float synth_gain;             // random weights: N(0, gain^2 / ne0); < 0: 1 + 0.1 N(0, 1) (norm weights)
+};
+
+static bool parse_nigozen_config(const json_value & cfg, llm_model * m, std::string & err) {
+    llm_hparams & hp = m->hp;
+    snprintf(hp.arch, sizeof(hp.arch), "nigozen");
+    const json_value * layers = cfg.get("layers");
+    if (!layers || layers->kind != json_value::ARR || layers->arr.empty()) { err = "config: no layers"; return false; }
+    const json_value * v;
+    hp.n_embd = (v = cfg.get("width")) ? (int) v->number(0) : 0;
+    hp.n_vocab = (v = cfg.get("vocab")) ? (int) v->number(0) : 0;
+    hp.rms_eps = (v = cfg.path("norm", "eps")) ? (float) v->number(1e-5) : 1e-5f;
+    m->embd_scale = (v = cfg.path("embedding", "scale")) ? (float) v->number(1.0) : 1.0f;
+    hp.n_layer = (int) layers->arr.size();
+    hp.n_ctx_train = 1 << 20;
+    if (hp.n_embd <= 0 || hp.n_vocab <= 0) { err = "config: width / vocab missing"; return false; }
+    m->lcfg.resize((size_t) hp.n_layer);
+    for (int il = 0; il < hp.n_layer; ++il) {
+        const json_value & L = layers->arr[(size_t) il];
+        llm_layer_cfg & c = m->lcfg[(size_t) il];
+        const json_value * type = L.get("type");
+        if (!type || type->kind != json_value::STR || type->str != "attention") { err = "config: layer " + std::to_string(il) + ": unknown mixer type"; return false; }
+        const json_value * mx = L.get("mixer");
+        if (!mx || mx->kind != json_value::OBJ) { err = "config: layer without a mixer"; return false; }
+        auto num = [&](const json_value * o, const char * k0, const char * k1, double d) { const json_value * x = o->path(k0, k1); return x ? x->number(d) : d; };
+        c.n_head = (int) num(mx, "heads", nullptr, 0);
+        c.n_head_kv = (int) num(mx, "kv_heads", nullptr, c.n_head);
+        c.dk = (int) num(mx, "dim", nullptr, 0);
+        c.dv = (int) num(mx, "vdim", nullptr, c.dk);
+        c.rot_dims = (int) num(mx, "rot", "dims", 0);
+        c.rot_base = (float) num(mx, "rot", "base", 10000.0);
+        c.scale = (float) num(mx, "scale", nullptr, c.dk > 0 ? 1.0 / sqrt((double) c.dk) : 1.0);
+        c.chunk = (int) num(mx, "mask", "size", 0);
+        c.v_mix = num(mx, "v_mix", nullptr, 0) != 0;
+        c.sink = true;      // the design's soft-max always carries the sink ...
+        c.out_gate = true;  // ... and its heads always pass the sigmoid gate
+        if (c.n_head <= 0 || c.n_head_kv <= 0 || c.n_head % c.n_head_kv || c.dk <= 0 || c.dv <= 0 || c.rot_dims < 0 || c.rot_dims > c.dk || (c.rot_dims & 1) || c.chunk < 0) {
+            err = "config: layer " + std::to_string(il) + ": inconsistent attention sizes";
+            return false;
+        }
+        const json_value * ml = L.path("mlp");
+        if (ml) {
+            const json_value * kind = ml->get("kind");
+            if (kind && kind->kind == json_value::STR && kind->str == "dense") {
+                c.mlp = LLM_MLP_DENSE;
+                c.n_ff = (int) num(ml, "ff", nullptr, 0);
+            } else if (kind && kind->kind == json_value::STR && kind->str == "moe") {
+                c.mlp = LLM_MLP_MOE;
+                c.n_ff = (int) num(ml, "expert", "ff", 0);
+                c.n_expert = (int) num(ml, "router", "experts", 0);
+                c.n_top = (int) num(ml, "router", "top", 0);
+                if (c.n_expert <= 0 || c.n_top <= 0 || c.n_top > c.n_expert) { err = "config: layer " + std::to_string(il) + ": inconsistent router"; return false; }
+            } else { err = "config: layer " + std::to_string(il) + ": unknown mlp kind"; return false; }
+            if (c.n_ff <= 0) { err = "config: layer " + std::to_string(il) + ": ff missing"; return false; }
+        }
+        size_t k = 0;
+        while (k < m->mask_chunks.size() && m->mask_chunks[k] != c.chunk) ++k;
+        if (k == m->mask_chunks.size()) m->mask_chunks.push_back(c.chunk);
+        c.mask_id = (int) k;
+        m->max_embd_k = std::max(m->max_embd_k, c.n_head_kv * c.dk);
+        m->max_embd_v = std::max(m->max_embd_v, c.n_head_kv * c.dv);
+    }
+    // the uniform fields describe layer 0 (informational for per-layer models)
+    hp.n_head = m->lcfg[0].n_head; hp.n_head_kv = m->lcfg[0].n_head_kv; hp.n_embd_head = m->lcfg[0].dk; hp.n_ff = m->lcfg[0].n_ff;
+    hp.rope_freq_base = m->lcfg[0].rot_base;
+    return true;
+}
+
+static std::vector<dir_tensor> nigozen_plan(const llm_model * m) {
+    const llm_hparams & hp = m->hp;
+    const ggml_type wt = m->wtype;
+    const int64_t E = hp.n_embd;
+    std::vector<dir_tensor> plan;
+    auto add = [&](const std::string & name, ggml_type t, int64_t n0, int64_t n1, int64_t n2, std::vector<std::string> src, float gain) {
+        plan.push_back({name, t, {n0, n1, n2}, std::move(src), gain});
+    };
+    add("token_embd.weight", wt, E, hp.n_vocab, 1, {"embed"}, sqrtf((float) E));
+    int max_head = 1;
+    for (int il = 0; il < hp.n_layer; ++il) {
+        const llm_layer_cfg & c = m->lcfg[(size_t) il];
+        const std::string p = "blk." + std::to_string(il) + ".", q = "l" + std::to_string(il) + ".";
+        max_head = std::max(max_head, c.n_head);
+        add(p + "attn_norm.weight", GGML_TYPE_F32, E, 1, 1, {q + "norm1"}, -1.0f);
+        add(p + "attn_post_norm.weight", GGML_TYPE_F32, E, 1, 1, {q + "norm1b"}, -1.0f);
+        add(p + "attn_q.weight", wt, E, (int64_t) c.n_head * c.dk, 1, {q + "mix.q"}, 2.0f);
+        add(p + "attn_k.weight", wt, E, (int64_t) c.n_head_kv * c.dk, 1, {q + "mix.k"}, 2.0f);
+        add(p + "attn_v.weight", wt, E, (int64_t) c.n_head_kv * c.dv, 1, {q + "mix.v"}, 1.0f);
+        add(p + "attn_gate.weight", wt, E, (int64_t) c.n_head * c.dv, 1, {q + "mix.g"}, 1.0f);
+        add(p + "attn_output.weight", wt, (int64_t) c.n_head * c.dv, E, 1, {q + "mix.o"}, 1.0f);
+        if (c.mlp != LLM_MLP_NONE) {
+            add(p + "ffn_norm.weight", GGML_TYPE_F32, E, 1, 1, {q + "norm2"}, -1.0f);
+            add(p + "ffn_post_norm.weight", GGML_TYPE_F32, E, 1, 1, {q + "norm2b"}, -1.0f);
+        }
+        if (c.mlp == LLM_MLP_DENSE) {
+            add(p + "ffn_up.weight", wt, E, c.n_ff, 1, {q + "mlp.up"}, 1.0f);
+            add(p + "ffn_down.weight", wt, c.n_ff, E, 1, {q + "mlp.down"}, 1.0f);
+        } else if (c.mlp == LLM_MLP_MOE) {
+            std::vector<std::string> ups, downs;
+            for (int e = 0; e < c.n_expert; ++e) {
+                ups.push_back(q + "mlp.e" + std::to_string(e) + ".up");
+                downs.push_back(q + "mlp.e" + std::to_string(e) + ".down");
+            }
+            add(p + "ffn_gate_inp.weight", GGML_TYPE_F32, E, c.n_expert, 1, {q + "mlp.router"}, 3.0f);  // router logits are 32-bit in every mode
+            add(p + "ffn_up_exps.weight", wt, E, c.n_ff, c.n_expert, ups, 2.0f);
+            add(p + "ffn_down_exps.weight", wt, c.n_ff, E, c.n_expert, downs, 1.0f);
+        }
+    }
+    add("output_norm.weight", GGML_TYPE_F32, E, 1, 1, {"final.norm"}, -1.0f);
+    add("attn_sinks.weight", GGML_TYPE_F32, max_head, 1, 1, {}, 0.0f);
+    return plan;
+}
+
+// values of one checkpoint tensor (bf16 / f32 / f16 in the file) as `type` (bf16 or f32) into dst
+static bool convert_values(const st_tensor & t, ggml_type type, uint8_t * dst) {
+    const int64_t n = t.numel();
+    for (int64_t i = 0; i < n; ++i) {
+        float f;
+        if (t.dtype == "BF16") { uint16_t h; memcpy(&h, t.data + i * 2, 2); if (type == GGML_TYPE_BF16) { memcpy(dst + i * 2, &h, 2); continue; } f = bf16_to_f32(h); }
+        else if (t.dtype == "F32") memcpy(&f, t.data + i * 4, 4);
+        else if (t.dtype == "F16") { uint16_t h; memcpy(&h, t.data + i * 2, 2); f = f16_to_f32(h); }
+        else return false;
+        if (type == GGML_TYPE_F32) memcpy(dst + i * 4, &f, 4);
+        else { const uint16_t h = f32_to_bf16(f); memcpy(dst + i * 2, &h, 2); }
+    }
+    return true;
+}
+
+static float gauss(uint64_t & s) {  // Box-Muller on two uniforms
+    const float u1 = std::max(u01(splitmix64(s)), 1e-7f), u2 = u01(splitmix64(s));
+    return sqrtf(-2.0f * logf(u1)) * cosf(6.2831853f * u2);
+}
+
+static llm_model * model_from_config(const json_value & cfg, const st_file * file, uint64_t seed, ggml_backend_buffer_type_t buft, int wtype) {
+    const json_value * arch = cfg.get("architecture");
+    if (!arch || arch->kind != json_value::STR) { fprintf(stderr, "llm_model_load_dir: config.json names no architecture\n"); return nullptr; }
+    if (wtype != GGML_TYPE_BF16 && wtype != GGML_TYPE_F32) { fprintf(stderr, "llm_model_load_dir: matrices are kept as bf16 or f32\n"); return nullptr; }
+    llm_model * m = new llm_model();
+    m->wtype = (ggml_type) wtype;
+    std::string err;
+    // the registry of model classes that are described by a config.json
+    if (arch->str == "Nigozen") {
+        if (!parse_nigozen_config(cfg, m, err)) { fprintf(stderr, "llm_model_load_dir: %s\n", err.c_str()); delete m; return nullptr; }
+    } else {
+        fprintf(stderr, "llm_model_load_dir: unknown architecture \"%s\"\n", arch->str.c_str());
+        delete m;
+        return nullptr;
+    }
+    std::vector<dir_tensor> plan = nigozen_plan(m);
+    m->ctx = ggml_init({0, nullptr, true});
+    for (auto & t : plan) {
+        // shapes are checked against the file before anything is allocated
+        if (file)
+            for (auto & sname : t.src) {
+                const st_tensor * st = file->find(sname);
+                const int64_t want = t.ne[0] * t.ne[1];
+                if (!st || st->numel() != want || (st->shape.size() == 2 && (st->shape[1] != t.ne[0] || st->shape[0] != t.ne[1]))) {
+                    fprintf(stderr, "llm_model_load_dir: tensor %s is missing or has another shape than the config implies\n", sname.c_str());
+                    llm_model_free(m);
+                    return nullptr;
+                }
+            }
+        ggml_tensor * x = ggml_new_tensor_3d(m->ctx, t.type, t.ne[0], t.ne[1], t.ne[2]);
+        ggml_set_name(x, t.name.c_str());
+    }
+    ggml_backend_buffer_t buf = ggml_backend_alloc_ctx_tensors_from_buft(m->ctx, buft);
+    if (!buf) { fprintf(stderr, "llm_model_load_dir: failed to allocate weights\n"); llm_model_free(m); return nullptr; }
+    ggml_backend_buffer_set_usage(buf, GGML_BACKEND_BUFFER_USAGE_WEIGHTS);
+    m->buffers.push_back(buf);
+    std::vector<uint8_t> stage;
+    int tid = 0;
+    for (auto & t : plan) {
+        ggml_tensor * x = ggml_get_tensor(m->ctx, t.name.c_str());
+        const size_t esz = ggml_type_size(t.type), slice = (size_t) (t.ne[0] * t.ne[1]) * esz;
+        stage.assign(slice * (size_t) t.ne[2], 0);
+        ++tid;
+        if (t.src.empty()) {
+            // zeros (the sinks)
+        } else if (file) {
+            for (size_t k = 0; k < t.src.size(); ++k)
+                if (!convert_values(*file->find(t.src[k]), t.type, stage.data() + k * slice)) {
+                    fprintf(stderr, "llm_model_load_dir: tensor %s has an unsupported dtype\n", t.src[k].c_str());
+                    llm_model_free(m);
+                    return nullptr;
+                }
+        } else {
+            uint64_t s = seed ^ ((uint64_t) tid * 0xD1B54A32D192ED03ull);
+            const int64_t n = t.ne[0] * t.ne[1] * t.ne[2];
+            const float g = t.synth_gain / sqrtf((float) t.ne[0]);
+            for (int64_t i = 0; i < n; ++i) {
+                const float f = t.synth_gain < 0.0f ? 1.0f + 0.1f * gauss(s) : g * gauss(s);
+                if (t.type == GGML_TYPE_F32) memcpy(stage.data() + i * 4, &f, 4);
+                else { const uint16_t h = f32_to_bf16(f); memcpy(stage.data() + i * 2, &h, 2); }
+            }
+        }
+        ggml_backend_tensor_set(x, stage.data(), 0, stage.size());
+        m->total_bytes += stage.size();
+    }
+    // bind
+    m->tok_embd = ggml_get_tensor(m->ctx, "token_embd.weight");
+    m->output = m->tok_embd;  // the output matrix is the embedding table itself
+    m->output_norm = ggml_get_tensor(m->ctx, "output_norm.weight");
+    m->attn_sinks = ggml_get_tensor(m->ctx, "attn_sinks.weight");
+    m->layers.resize((size_t) m->hp.n_layer);
+    uint64_t sbytes = ggml_nbytes(m->tok_embd) + ggml_nbytes(m->output_norm);
+    for (int il = 0; il < m->hp.n_layer; ++il) {
+        const std::string p = "blk." + std::to_string(il) + ".";
+        auto g = [&](const char * s) { return ggml_get_tensor(m->ctx, (p + s).c_str()); };
+        llm_layer & L = m->layers[(size_t) il];
+        llm_layer_cfg & c = m->lcfg[(size_t) il];
+        L.attn_norm = g("attn_norm.weight"); L.attn_post_norm = g("attn_post_norm.weight"); L.wq = g("attn_q.weight"); L.wk = g("attn_k.weight");
+        L.wv = g("attn_v.weight"); L.attn_gate = g("attn_gate.weight"); L.wo = g("attn_output.weight");
+        L.ffn_norm = g("ffn_norm.weight"); L.ffn_post_norm = g("ffn_post_norm.weight"); L.ffn_up = g("ffn_up.weight"); L.ffn_down = g("ffn_down.weight");
+        L.ffn_gate_inp = g("ffn_gate_inp.weight"); L.ffn_up_exps = g("ffn_up_exps.weight"); L.ffn_down_exps = g("ffn_down_exps.weight");
+        for (ggml_tensor * t : {L.attn_norm, L.attn_post_norm, L.wq, L.wk, L.wv, L.attn_gate, L.wo, L.ffn_norm, L.ffn_post_norm, L.ffn_up, L.ffn_down, L.ffn_gate_inp})
+            if (t) sbytes += ggml_nbytes(t);
+        if (c.mlp == LLM_MLP_MOE) sbytes += (ggml_nbytes(L.ffn_up_exps) + ggml_nbytes(L.ffn_down_exps)) / (uint64_t) c.n_expert * (uint64_t) c.n_top;
+        if (c.v_mix) {  // the blend factor is a scalar of the checkpoint, read once
+            float lam = 0.5f;
+            if (file) {
+                const st_tensor * st = file->find("l" + std::to_string(il) + ".mix.vmix");
+                if (!st || st->numel() != 1) { fprintf(stderr, "llm_model_load_dir: layer %d has no scalar mix.vmix\n", il); llm_model_free(m); return nullptr; }
+                uint8_t tmp[4];
+                if (!convert_values(*st, GGML_TYPE_F32, tmp)) { llm_model_free(m); return nullptr; }
+                memcpy(&lam, tmp, 4);
+            } else {
+                uint64_t s = seed ^ (0xABCDull + (uint64_t) il);
+                lam = bf16_to_f32(f32_to_bf16(0.2f + 0.6f * u01(splitmix64(s))));
+            }
+            c.v_lambda = lam;
+        }
+    }
+    m->stream_bytes = sbytes;
+    m->n_head_l = m->hp.n_head; m->n_head_kv_l = m->hp.n_head_kv; m->n_ff_l = m->hp.n_ff;
+    m->n_vocab_l = m->hp.n_vocab;
+    return m;
+}
+
+extern "C" struct llm_model * llm_model_load_dir(const char * dir, ggml_backend_buffer_type_t buft, int wtype) {
+    const std::string d = dir;
+    std::string text;
+    {
+        FILE * f = fopen((d + "/config.json").c_str(), "rb");
+        if (!f) { fprintf(stderr, "llm_model_load_dir: %s/config.json cannot be read\n", dir); return nullptr; }
+        char buf[65536];
+        size_t n;
+        while ((n = fread(buf, 1, sizeof(buf), f)) > 0) text.append(buf, n);
+        fclose(f);
+    }
+    json_value cfg;
+    if (!json_parser::parse(text.data(), text.size(), cfg) || cfg.kind != json_value::OBJ) { fprintf(stderr, "llm_model_load_dir: %s/config.json is not a JSON object\n", dir); return nullptr; }
+    st_file * file = st_file::open((d + "/model.safetensors").c_str());
+    if (!file) return nullptr;
+    llm_model * m = model_from_config(cfg, file, 0, buft, wtype);
+    delete file;
+    return m;
+}
+extern "C" struct llm_model * llm_model_synth_config(const char * config_json, uint64_t seed, ggml_backend_buffer_type_t buft, int wtype) {
+    json_value cfg;
+    if (!config_json || !json_parser::parse(config_json, strlen(config_json), cfg) || cfg.kind != json_value::OBJ) { fprintf(stderr, "llm_model_synth_config: the text is not a JSON object\n"); return nullptr; }
+    return model_from_config(cfg, nullptr, seed, buft, wtype);
+}
+
 extern "C" void llm_model_free(struct llm_model * m) {
     if (!m) return;
     for (auto b : m->buffers) ggml_backend_buffer_free(b);
@@ -719,6 +1030,17 @@ static void mask_row(float * __restrict__ row, const int n_kv, const int32_t * _
         row[j] = v ? vis : hid;
     }
 }
+// the same with attention confined to chunks of `chunk` positions counted from position 0 of the sequence: cell j is visible to position p only when
+// floor(pos_j / chunk) == floor(p / chunk) as well (where a prompt was cut for processing plays no part: the rule reads positions only)
+static void mask_row_chunked(float * __restrict__ row, const int n_kv, const int32_t * __restrict__ cpos, const int32_t * __restrict__ cseq, const int32_t s, const int32_t p,
+                             const int32_t chunk, const float vis, const float hid) {
+    const int32_t lo = p / chunk * chunk;  // first position of p's chunk
+    const uint32_t span = (uint32_t) (p - lo);
+    for (int j = 0; j < n_kv; ++j) {
+        const bool v = (cseq[j] == s) & ((uint32_t) (cpos[j] - lo) <= span);  // lo <= pos_j <= p (an empty cell's -1 wraps to a huge value)
+        row[j] = v ? vis : hid;
+    }
+}
 #pragma GCC pop_options
 
 struct kv_cell {
@@ -731,6 +1053,7 @@ struct kv_cell {
 struct seg_io {
     ggml_tensor *tokens = nullptr, *pos = nullptr, *mask = nullptr, *k_idxs = nullptr, *v_idxs = nullptr, *out_ids = nullptr, *resid = nullptr;
     ggml_tensor * out = nullptr;  // l_out of the segment's last layer, or the logits
+    std::vector<ggml_tensor *> masks;  // models whose layers differ in what they may see: one mask per distinct rule (masks[0] == mask)
 };
 
 struct graph_key {
@@ -758,6 +1081,7 @@ struct llm_context {
     ggml_cgraph * gf = nullptr;
     graph_key key;
     ggml_tensor *inp_tokens = nullptr, *inp_pos = nullptr, *inp_mask = nullptr, *inp_k_idxs = nullptr, *inp_v_idxs = nullptr, *inp_out_ids = nullptr;
+    std::vector<ggml_tensor *> inp_masks;  // all masks of the graph (inp_masks[0] == inp_mask)
     ggml_tensor * t_logits = nullptr;
     // outputs
     std::vector<float> logits;
@@ -812,6 +1136,7 @@ static void make_inputs(llm_context * c, ggml_context * ctx, int l0, int l1, boo
     const llm_hparams & hp = m->hp;
     const bool fa = c->p.flash_attn != 0;
     const int64_t n_embd_k = (int64_t) m->n_head_kv_l * hp.n_embd_head;
+    io = seg_io();
     if (l0 == 0) {
         io.tokens = ggml_new_tensor_1d(ctx, GGML_TYPE_I32, n_tokens);
         ggml_set_input(named(io.tokens, "inp_tokens", -1));
@@ -826,6 +1151,11 @@ static void make_inputs(llm_context * c, ggml_context * ctx, int l0, int l1, boo
     // ggml_cast(F16) of it (self_kq_mask_cnv) — a CPY node in the graph, not an F16 upload
     io.mask = ggml_new_tensor_2d(ctx, GGML_TYPE_F32, n_kv, n_tok_pad);
     ggml_set_input(named(io.mask, "KQ_mask", -1));
+    io.masks.assign(1, io.mask);
+    for (size_t k = 1; k < m->mask_chunks.size(); ++k) {
+        io.masks.push_back(ggml_new_tensor_2d(ctx, GGML_TYPE_F32, n_kv, n_tok_pad));
+        ggml_set_input(named(io.masks.back(), "KQ_mask_chunked", (int) k));
+    }
     io.k_idxs = ggml_new_tensor_1d(ctx, GGML_TYPE_I64, n_tokens);
     ggml_set_input(named(io.k_idxs, "k_idxs", -1));
     if (!fa) {
@@ -925,13 +1255,119 @@ static void build_segment(llm_context * c, ggml_context * ctx, ggml_cgraph * gf,
     io.out = cur;
 }
 
+// The graph of a model described layer by layer (llm_layer_cfg).  Per layer, with h the normed input:
+//   q, k = rope(W_q h), rope(W_k h) on the leading rot_dims of every head; v = W_v h, blended with the first value-mixing layer's v;
+//   k, v -> cache; attention over the cache under the layer's mask, soft-max with a sink; heads x sigmoid(W_g h); W_o; norm; + residual;
+//   then the feed-forward (dense erf-GELU, or top-k experts with squared ReLU), normed before and after; + residual.
+// Layer norms are NORM x weight; the residual stream and everything around the mat-muls stays f32.
+static ggml_tensor * layer_norm_w(ggml_context * ctx, ggml_tensor * x, ggml_tensor * w, float eps, const char * name, int il) {
+    ggml_tensor * n = named(ggml_norm(ctx, x, eps), "lnorm", il);
+    return named(ggml_mul(ctx, n, w), name, il);
+}
+
+static ggml_tensor * build_moe(ggml_context * ctx, ggml_cgraph * gf, const llm_layer & L, const llm_layer_cfg & c, ggml_tensor * cur, int il) {
+    const int64_t E = cur->ne[0], T = cur->ne[1];
+    ggml_tensor * logits = named(ggml_mul_mat(ctx, L.ffn_gate_inp, cur), "ffn_moe_logits", il);  // [n_expert, T], f32 weights: 32-bit
+    ggml_tensor * sel = named(ggml_top_k(ctx, logits, c.n_top), "ffn_moe_topk", il);            // [n_top, T] i32
+    ggml_tensor * w = ggml_get_rows(ctx, ggml_reshape_3d(ctx, logits, 1, c.n_expert, T), sel);   // [1, n_top, T]
+    w = named(ggml_soft_max(ctx, ggml_reshape_2d(ctx, named(w, "ffn_moe_sel_logits", il), c.n_top, T)), "ffn_moe_weights", il);  // soft-max over the chosen logits only
+    ggml_tensor * up = named(ggml_mul_mat_id(ctx, L.ffn_up_exps, ggml_reshape_3d(ctx, cur, E, 1, T), sel), "ffn_moe_up", il);     // [n_ff, n_top, T]
+    ggml_tensor * act = named(ggml_sqr(ctx, named(ggml_unary(ctx, up, GGML_UNARY_OP_RELU), "ffn_moe_relu", il)), "ffn_moe_act", il);
+    ggml_tensor * down = named(ggml_mul_mat_id(ctx, L.ffn_down_exps, act, sel), "ffn_moe_down", il);                              // [E, n_top, T]
+    down = named(ggml_mul(ctx, down, ggml_reshape_3d(ctx, w, 1, c.n_top, T)), "ffn_moe_weighted", il);
+    ggml_build_forward_expand(gf, down);
+    ggml_tensor * out = nullptr;
+    for (int j = 0; j < c.n_top; ++j) {  // the sum over the chosen experts, as a chain of adds over views
+        ggml_tensor * v = ggml_view_2d(ctx, down, E, T, down->nb[2], (size_t) j * down->nb[1]);
+        out = out ? ggml_add(ctx, out, v) : v;
+    }
+    if (c.n_top == 1) out = ggml_cont(ctx, out);
+    return named(out, "ffn_moe_out", il);
+}
+
+static void build_layerwise(llm_context * c, ggml_context * ctx, ggml_cgraph * gf, int n_tokens, int n_kv, seg_io & io) {
+    llm_model * m = c->model;
+    const llm_hparams & hp = m->hp;
+    const float eps = hp.rms_eps;
+    std::vector<ggml_tensor *> mask_cnv;
+    for (size_t k = 0; k < io.masks.size(); ++k) mask_cnv.push_back(named(ggml_cast(ctx, io.masks[k], GGML_TYPE_F16), "KQ_mask_cnv", (int) k));
+    ggml_tensor * inpL = named(ggml_get_rows(ctx, m->tok_embd, io.tokens), "inp_embd", -1);
+    if (m->embd_scale != 1.0f) inpL = named(ggml_scale(ctx, inpL, m->embd_scale), "inp_scaled", -1);
+    ggml_tensor * v_first = nullptr;
+    for (int il = 0; il < hp.n_layer; ++il) {
+        const llm_layer & L = m->layers[(size_t) il];
+        const llm_layer_cfg & lc = m->lcfg[(size_t) il];
+        const int64_t H = lc.n_head, G = lc.n_head_kv, DK = lc.dk, DV = lc.dv;
+        ggml_tensor * inpSA = inpL;
+        ggml_tensor * cur = layer_norm_w(ctx, inpL, L.attn_norm, eps, "attn_norm", il);
+        ggml_tensor * Qcur = named(ggml_mul_mat(ctx, L.wq, cur), "Qcur", il);
+        ggml_tensor * Kcur = named(ggml_mul_mat(ctx, L.wk, cur), "Kcur", il);
+        ggml_tensor * Vcur = named(ggml_mul_mat(ctx, L.wv, cur), "Vcur", il);
+        ggml_tensor * gate = lc.out_gate ? named(ggml_mul_mat(ctx, L.attn_gate, cur), "attn_gate", il) : nullptr;
+        Qcur = ggml_reshape_3d(ctx, Qcur, DK, H, n_tokens);
+        Kcur = ggml_reshape_3d(ctx, Kcur, DK, G, n_tokens);
+        if (lc.rot_dims > 0) {  // neighbouring pairs (2i, 2i + 1) of the leading rot_dims entries; the rest of the head passes through
+            Qcur = named(ggml_rope_ext(ctx, Qcur, io.pos, nullptr, lc.rot_dims, 0, hp.n_ctx_train, lc.rot_base, 1.0f, 0.0f, 1.0f, 32.0f, 1.0f), "Qcur_rope", il);
+            Kcur = named(ggml_rope_ext(ctx, Kcur, io.pos, nullptr, lc.rot_dims, 0, hp.n_ctx_train, lc.rot_base, 1.0f, 0.0f, 1.0f, 32.0f, 1.0f), "Kcur_rope", il);
+        }
+        if (lc.v_mix) {
+            if (!v_first) v_first = Vcur;
+            else {
+                LLM_ASSERT(v_first->ne[0] == Vcur->ne[0]);
+                Vcur = named(ggml_add(ctx, named(ggml_scale(ctx, Vcur, 1.0f - lc.v_lambda), "Vcur_own", il), named(ggml_scale(ctx, v_first, lc.v_lambda), "Vcur_first", il)), "Vcur_mixed", il);
+            }
+        }
+        ggml_build_forward_expand(gf, Qcur);
+        ggml_build_forward_expand(gf, Kcur);
+        ggml_build_forward_expand(gf, Vcur);
+        ggml_tensor * k_cache = c->k_l[(size_t) il];
+        ggml_tensor * v_cache = c->v_l[(size_t) il];
+        ggml_build_forward_expand(gf, named(ggml_set_rows(ctx, k_cache, ggml_reshape_2d(ctx, Kcur, G * DK, n_tokens), io.k_idxs), "k_store", il));
+        ggml_build_forward_expand(gf, named(ggml_set_rows(ctx, v_cache, ggml_reshape_2d(ctx, Vcur, G * DV, n_tokens), io.k_idxs), "v_store", il));  // the blended values are what is kept
+        ggml_tensor * q = ggml_permute(ctx, Qcur, 0, 2, 1, 3);
+        ggml_tensor * k = ggml_view_3d(ctx, k_cache, DK, n_kv, G, ggml_row_size(k_cache->type, G * DK), ggml_row_size(k_cache->type, DK), 0);
+        ggml_tensor * v = ggml_view_3d(ctx, v_cache, DV, n_kv, G, ggml_row_size(v_cache->type, G * DV), ggml_row_size(v_cache->type, DV), 0);
+        cur = ggml_flash_attn_ext(ctx, q, k, v, mask_cnv[(size_t) lc.mask_id], lc.scale, 0.0f, 0.0f);
+        ggml_flash_attn_ext_set_prec(cur, GGML_PREC_F32);
+        if (lc.sink) ggml_flash_attn_ext_add_sinks(cur, ggml_view_1d(ctx, m->attn_sinks, H, 0));
+        named(cur, "fattn", il);
+        cur = ggml_reshape_2d(ctx, cur, DV * H, n_tokens);
+        if (gate) cur = named(ggml_mul(ctx, cur, named(ggml_unary(ctx, gate, GGML_UNARY_OP_SIGMOID), "attn_gate_sigmoid", il)), "attn_gated", il);
+        cur = named(ggml_mul_mat(ctx, L.wo, cur), "attn_out", il);
+        if (il == hp.n_layer - 1 && io.out_ids) {  // only the rows whose logits are wanted go on from here
+            cur = ggml_get_rows(ctx, cur, io.out_ids);
+            inpSA = ggml_get_rows(ctx, inpSA, io.out_ids);
+        }
+        cur = layer_norm_w(ctx, cur, L.attn_post_norm, eps, "attn_post_norm", il);
+        ggml_tensor * ffn_inp = named(ggml_add(ctx, cur, inpSA), lc.mlp == LLM_MLP_NONE ? "l_out" : "ffn_inp", il);
+        if (lc.mlp == LLM_MLP_NONE) { inpL = ffn_inp; continue; }
+        cur = layer_norm_w(ctx, ffn_inp, L.ffn_norm, eps, "ffn_norm", il);
+        if (lc.mlp == LLM_MLP_DENSE) {
+            cur = named(ggml_mul_mat(ctx, L.ffn_up, cur), "ffn_up", il);
+            cur = named(ggml_unary(ctx, cur, GGML_UNARY_OP_GELU_ERF), "ffn_gelu", il);
+            cur = named(ggml_mul_mat(ctx, L.ffn_down, cur), "ffn_out", il);
+        } else {
+            cur = build_moe(ctx, gf, L, lc, cur, il);
+        }
+        cur = layer_norm_w(ctx, cur, L.ffn_post_norm, eps, "ffn_post_norm", il);
+        inpL = named(ggml_add(ctx, cur, ffn_inp), "l_out", il);
+    }
+    ggml_tensor * cur = layer_norm_w(ctx, inpL, m->output_norm, eps, "result_norm", -1);
+    cur = named(ggml_mul_mat(ctx, m->output, cur), "result_output", -1);
+    ggml_set_output(cur);
+    ggml_build_forward_expand(gf, cur);
+    io.out = cur;
+}
+
 static void build_graph(llm_context * c, int n_tokens, int n_kv, int n_outputs) {
     if (c->ctx_compute) ggml_free(c->ctx_compute);
     c->ctx_compute = ggml_init({0, nullptr, true});
     ggml_cgraph * gf = ggml_new_graph_custom(c->ctx_compute, 8192, false);
     seg_io io;
     make_inputs(c, c->ctx_compute, 0, c->model->hp.n_layer, true, n_tokens, n_kv, n_outputs, io);
-    build_segment(c, c->ctx_compute, gf, 0, c->model->hp.n_layer, true, n_tokens, n_kv, io);
+    if (!c->model->lcfg.empty()) build_layerwise(c, c->ctx_compute, gf, n_tokens, n_kv, io);
+    else build_segment(c, c->ctx_compute, gf, 0, c->model->hp.n_layer, true, n_tokens, n_kv, io);
+    c->inp_masks = io.masks;
     c->inp_tokens = io.tokens;
     c->inp_pos = io.pos;
     c->inp_mask = io.mask;
@@ -965,7 +1401,15 @@ extern "C" struct llm_context * llm_context_new(struct llm_model * m, ggml_backe
         return t == GGML_TYPE_F32 || t == GGML_TYPE_F16 || t == GGML_TYPE_BF16 || t == GGML_TYPE_Q8_0 || t == GGML_TYPE_Q4_0 || t == GGML_TYPE_Q4_1 || t == GGML_TYPE_IQ4_NL ||
                t == GGML_TYPE_Q5_0 || t == GGML_TYPE_Q5_1;
     };
-    const ggml_type type_k = kv_type_of(c->p.type_k), type_v = kv_type_of(c->p.type_v);
+    // a model described layer by layer runs its attention as one fused op over a cache kept, by default, in the type of its matrices (bf16 or f32)
+    const bool layerwise = !m->lcfg.empty();
+    if (layerwise) c->p.flash_attn = 1;
+    const ggml_type type_k = (layerwise && c->p.type_k == 0) ? m->wtype : kv_type_of(c->p.type_k), type_v = (layerwise && c->p.type_v == 0) ? m->wtype : kv_type_of(c->p.type_v);
+    if (layerwise && (ggml_blck_size(type_k) != 1 || ggml_blck_size(type_v) != 1)) {
+        fprintf(stderr, "llm_context_new: a per-layer model keeps its cache in f32, f16 or bf16\n");
+        delete c;
+        return nullptr;
+    }
     // (llama.cpp: a quantised V cache needs flash attention — the non-flash path keeps V transposed, one element per index; K may be of any type there:
     // K.q is then a MUL_MAT over the cache's blocks)
     if (!kv_type_ok(type_k) || !kv_type_ok(type_v) || (type_v != GGML_TYPE_F16 && !c->p.flash_attn) || (hp.n_embd_head % ggml_blck_size(type_k)) != 0 || (hp.n_embd_head % ggml_blck_size(type_v)) != 0) {
@@ -975,8 +1419,11 @@ extern "C" struct llm_context * llm_context_new(struct llm_model * m, ggml_backe
     }
     c->ctx_kv = ggml_init({0, nullptr, true});
     for (int il = 0; il < hp.n_layer; ++il) {
-        ggml_tensor * k = ggml_new_tensor_2d(c->ctx_kv, type_k, n_embd_k, c->p.n_ctx);
-        ggml_tensor * v = c->p.flash_attn ? ggml_new_tensor_2d(c->ctx_kv, type_v, n_embd_k, c->p.n_ctx)
+        // (a model described layer by layer: every layer's cache rows have that layer's own widths, K and V apart)
+        const int64_t row_k = layerwise ? (int64_t) m->lcfg[(size_t) il].n_head_kv * m->lcfg[(size_t) il].dk : n_embd_k;
+        const int64_t row_v = layerwise ? (int64_t) m->lcfg[(size_t) il].n_head_kv * m->lcfg[(size_t) il].dv : n_embd_k;
+        ggml_tensor * k = ggml_new_tensor_2d(c->ctx_kv, type_k, row_k, c->p.n_ctx);
+        ggml_tensor * v = c->p.flash_attn ? ggml_new_tensor_2d(c->ctx_kv, type_v, row_v, c->p.n_ctx)
                                           : ggml_new_tensor_2d(c->ctx_kv, GGML_TYPE_F16, c->p.n_ctx, n_embd_k);
         named(k, "cache_k_l", il);
         named(v, "cache_v_l", il);
@@ -1006,7 +1453,7 @@ extern "C" struct llm_context * llm_context_new(struct llm_model * m, ggml_backe
         if (hbuft) {
             const size_t nub = (size_t) std::min(c->p.n_ubatch, c->p.n_ctx);
             const size_t n_tok_pad = (nub + 63) / 64 * 64;
-            size_t in_bytes = nub * (4 + 4 + 8 + 4) + n_tok_pad * (size_t) c->p.n_ctx * 4 + 256;
+            size_t in_bytes = nub * (4 + 4 + 8 + 4) + std::max<size_t>(1, m->mask_chunks.size()) * (n_tok_pad * (size_t) c->p.n_ctx * 4 + 64) + 256;
             if (!c->p.flash_attn) in_bytes += nub * (size_t) n_embd_k * 8;
             in_bytes = (in_bytes + 255) / 256 * 256;
             c->pin_out_rows = 64;
@@ -1395,11 +1842,17 @@ static int decode_ubatch(llm_context * c, int n_tokens, const int32_t * tokens, 
             cpos[j] = c->cells[j].pos;
             cseq[j] = c->cells[j].seq;
         }
-        upload(c->inp_mask, (size_t) n_kv * rows * 4, [&](char * d) {
-            float * mask = (float *) d;
-            for (size_t e = (size_t) n_kv * n_tokens; e < (size_t) n_kv * rows; ++e) mask[e] = -INFINITY;
-            for (int i = 0; i < n_tokens; ++i) mask_row(mask + (size_t) i * n_kv, n_kv, cpos.data(), cseq.data(), seq_id ? seq_id[i] : 0, pos[i], 0.0f, -INFINITY);
-        });
+        for (size_t mk = 0; mk < c->inp_masks.size(); ++mk) {
+            const int chunk = mk < m->mask_chunks.size() ? m->mask_chunks[mk] : 0;
+            upload(c->inp_masks[mk], (size_t) n_kv * rows * 4, [&](char * d) {
+                float * mask = (float *) d;
+                for (size_t e = (size_t) n_kv * n_tokens; e < (size_t) n_kv * rows; ++e) mask[e] = -INFINITY;
+                for (int i = 0; i < n_tokens; ++i) {
+                    if (chunk > 0) mask_row_chunked(mask + (size_t) i * n_kv, n_kv, cpos.data(), cseq.data(), seq_id ? seq_id[i] : 0, pos[i], chunk, 0.0f, -INFINITY);
+                    else mask_row(mask + (size_t) i * n_kv, n_kv, cpos.data(), cseq.data(), seq_id ? seq_id[i] : 0, pos[i], 0.0f, -INFINITY);
+                }
+            });
+        }
     }
     const double t2 = now_us();
     const size_t logit_bytes = (size_t) n_outputs * m->n_vocab_l * 4;

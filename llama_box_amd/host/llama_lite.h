@@ -58,6 +58,14 @@ struct llm_model * llm_model_synth_split(const struct llm_hparams * hp, uint64_t
 struct llm_model * llm_model_synth_layer_split(const struct llm_hparams * hp, uint64_t seed, const ggml_backend_buffer_type_t * bufts, int n_dev);
 int llm_synth_gguf(const struct llm_hparams * hp, uint64_t seed, const char * path);
 struct llm_model * llm_model_load(const char * path, ggml_backend_buffer_type_t buft);
+/* A checkpoint FOLDER: config.json + model.safetensors.  config.json's "architecture" chooses the model class; today "Nigozen": a decoder whose
+ * layers are listed one by one in the config (grouped-query attention with partial interleaved rotary positions, attention confined to chunks of
+ * positions, a soft-max with a zero-score sink, value mixing with the first such layer, a sigmoid output gate, layer norms before and after every
+ * sublayer, a dense erf-GELU or a top-k mixture-of-experts feed-forward, tied output matrix).  wtype: GGML_TYPE_BF16 keeps the matrices as stored
+ * (bf16 products, f32 accumulation); GGML_TYPE_F32 widens them at load (everything in 32-bit).  Norm weights and routers are always f32. */
+struct llm_model * llm_model_load_dir(const char * dir, ggml_backend_buffer_type_t buft, int wtype);
+/* the same model classes from the TEXT of a config.json and seeded random weights (benchmarks at sizes no file exists for) */
+struct llm_model * llm_model_synth_config(const char * config_json, uint64_t seed, ggml_backend_buffer_type_t buft, int wtype);
 void llm_model_free(struct llm_model * m);
 const struct llm_hparams * llm_model_hparams(const struct llm_model * m);
 /* bytes of weights one decoded token streams (all matmul weights + norms + one token_embd row): SURVEY.md §8d */
