@@ -243,6 +243,8 @@ static void attn_f32_launch_t(hipStream_t s, const tdesc & q, const tdesc & k, c
         const dim3 grid((unsigned) ((n_q + 63) / 64), (unsigned) H);
         auto go = [&](auto kern, int dkp, int dvp) {
             const size_t lds = ((size_t) 64 * (dkp + 1) + (size_t) 64 * dvp + (size_t) 64 * dkp) * sizeof(float);
+            // (more than the 64 KB a kernel gets by default: up to 97 KB of the CU's 160 KB; the attribute is per device and cheap to set again)
+            if (lds > 48 * 1024) (void) hipFuncSetAttribute((const void *) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds);
             hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, q, k, v, *mask, sinks, dst, scale);
         };
         const bool k64 = DK <= 64, v64 = DV <= 64;

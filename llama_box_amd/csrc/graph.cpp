@@ -109,6 +109,9 @@ static int fa_route(const ggml_tensor * op) {
     return (k16 && v16) ? 1 : 3;
 }
 
+// f32 rows that kv_types.hip can turn into bf16 a block of 32 values at a time (whole blocks, 16-byte aligned rows); others go element by element
+static bool bf16_rows_in_blocks(const ggml_tensor * a) { return (a->ne[0] % 32) == 0 && (a->nb[1] % 16) == 0 && (a->nb[2] % 16) == 0 && (a->nb[3] % 16) == 0; }
+
 bool supports_op(const ggml_tensor * op) {
     const ggml_tensor * a = op->src[0];
     const ggml_tensor * b = op->src[1];
@@ -172,7 +175,7 @@ bool supports_op(const ggml_tensor * op) {
             return b->type == GGML_TYPE_I32 && op->type == GGML_TYPE_F32 && rows_contig(a) && op->nb[0] == 4 &&
                    (is_quant(a->type) || a->type == GGML_TYPE_F16 || a->type == GGML_TYPE_F32 || a->type == GGML_TYPE_BF16);
         case GGML_OP_SET_ROWS:
-            if (op->type == GGML_TYPE_BF16 && (a->ne[0] % 32) != 0)  // bf16 rows that are not whole groups of 32 values: the element-wise form (ops.hip)
+            if (op->type == GGML_TYPE_BF16 && !bf16_rows_in_blocks(a))  // bf16 rows that are not whole, aligned groups of 32 values: the element-wise form (ops.hip)
                 return a->type == GGML_TYPE_F32 && b->type == GGML_TYPE_I64 && a->nb[0] == 4 && op->nb[0] == 2;
             if (kv_store_type(op->type))  // a cache row in q4_0 / q4_1 / q5_0 / q5_1 / iq4_nl / bf16: the type's from_float per block of 32 (kv_types.hip)
                 return a->type == GGML_TYPE_F32 && b->type == GGML_TYPE_I64 && a->nb[0] == 4 && (a->ne[0] % 32) == 0 && (a->nb[1] % 16) == 0 && (a->nb[2] % 16) == 0 && (a->nb[3] % 16) == 0 &&
@@ -2084,12 +2087,12 @@ static int run_node(exec_state & st, int i) {
         case GGML_OP_SET_ROWS: {
             timed_scope ts(c, "set_rows", (double) ggml_abi_nbytes(a));
             if (n->type == GGML_TYPE_Q8_0) launch_set_rows_q8_0(s, TD(a), TD(b), TD(n));
-            else if (kv_store_type(n->type) && !(n->type == GGML_TYPE_BF16 && (a->ne[0] % 32) != 0)) {
+            else if (kv_store_type(n->type) && !(n->type == GGML_TYPE_BF16 && !bf16_rows_in_blocks(a))) {
                 // K and V rows of a step go into their caches through the same indices: SET_ROWS(k), [views], SET_ROWS(v) as ONE launch
                 int j = i + 1;
                 while (j < g->n_nodes && (st.done[j] || is_view_op(g->nodes[j]))) ++j;
                 const ggml_tensor * n2 = j < g->n_nodes ? g->nodes[j] : nullptr;
-                if (fuse && n2 && n2->op == GGML_OP_SET_ROWS && kv_store_type(n2->type) && n2->src[0]->type == GGML_TYPE_F32 && n2->src[1]->type == GGML_TYPE_I64 &&
+                if (fuse && n2 && n2->op == GGML_OP_SET_ROWS && kv_store_type(n2->type) && !(n2->type == GGML_TYPE_BF16 && !bf16_rows_in_blocks(n2->src[0])) && n2->src[0]->type == GGML_TYPE_F32 && n2->src[1]->type == GGML_TYPE_I64 &&
                     n2->src[0] != n && !ranges_overlap(n2->src[0], n) && !ranges_overlap(n2, n) && supports_op(n2)) {
                     launch_set_rows_kv_pair(s, TD(a), TD(b), TD(n), TD(n2->src[0]), TD(n2->src[1]), TD(n2));
                     mark_done(st, j);

@@ -16,10 +16,14 @@ def preset(name, **over):
 
 
 class Model:
-    def __init__(self, hp=None, seed=1234, buft=None, path=None, tp_rank=0, tp_size=1, rowpar_buft=None, split_buft=None, layer_bufts=None):
+    def __init__(self, hp=None, seed=1234, buft=None, path=None, tp_rank=0, tp_size=1, rowpar_buft=None, split_buft=None, layer_bufts=None, folder=None, config_json=None, wtype=None):
         H = L.host()
         self.H = H
-        if layer_bufts is not None:  # -sm layer: device d's buffer type holds a contiguous range of layers
+        if folder is not None:  # a checkpoint folder: config.json + model.safetensors
+            self.m = H.llm_model_load_dir(folder.encode(), buft, L.BF16 if wtype is None else wtype)
+        elif config_json is not None:  # the same model classes with seeded random weights
+            self.m = H.llm_model_synth_config(config_json.encode(), seed, buft, L.BF16 if wtype is None else wtype)
+        elif layer_bufts is not None:  # -sm layer: device d's buffer type holds a contiguous range of layers
             arr = (C.c_void_p * len(layer_bufts))(*layer_bufts)
             self.m = H.llm_model_synth_layer_split(C.byref(hp), seed, arr, len(layer_bufts))
         elif path is not None:

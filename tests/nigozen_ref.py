@@ -108,8 +108,17 @@ def moe_ffn(h, W, p, ml):
     return out
 
 
-def forward(cfg, W, tokens, dtype=np.float64, return_layers=False):
-    """Whole-sequence forward of one request from position 0: logits [T, vocab] (and the residual stream after every layer)."""
+def router_margin(h, Wr, top):
+    """per token: gap between the last chosen and the first rejected router logit, in units of the logits' spread (inf when every expert is chosen)"""
+    z = np.sort(h @ Wr.T, axis=-1)[:, ::-1]
+    if top >= z.shape[1]:
+        return np.full(h.shape[0], np.inf)
+    return (z[:, top - 1] - z[:, top]) / (z.std(axis=-1) + 1e-30)
+
+
+def forward(cfg, W, tokens, dtype=np.float64, return_layers=False, margins=None):
+    """Whole-sequence forward of one request from position 0: logits [T, vocab] (and the residual stream after every layer).
+    margins: a list that receives, per mixture-of-experts layer, every token's router_margin."""
     W = {k: np.asarray(v, dtype=dtype) for k, v in W.items()}
     T = len(tokens)
     pos = np.arange(T)
@@ -127,7 +136,7 @@ def forward(cfg, W, tokens, dtype=np.float64, return_layers=False):
             if v_first is None:
                 v_first = v
             else:
-                v = mix_values(v, v_first, float(W[p + "mix.vmix"]))
+                v = mix_values(v.reshape(T, -1), v_first.reshape(T, -1), float(W[p + "mix.vmix"])).reshape(v.shape)  # per token, over all its value entries
         chunk = (mx.get("mask") or {}).get("size", 0)
         a = attend(q, k, v, pos, pos, mx["scale"], chunk)
         a = a * sigmoid(h @ W[p + "mix.g"].T)
@@ -136,6 +145,8 @@ def forward(cfg, W, tokens, dtype=np.float64, return_layers=False):
         if ml:
             h2 = layer_norm(x, W[p + "norm2"], eps)
             f = dense_ffn(h2, W, p) if ml["kind"] == "dense" else moe_ffn(h2, W, p, ml)
+            if margins is not None and ml["kind"] == "moe":
+                margins.append(router_margin(h2, W[p + "mlp.router"], ml["router"]["top"]))
             x = x + layer_norm(f, W[p + "norm2b"], eps)
         layers.append(x.copy())
     logits = layer_norm(x, W["final.norm"], eps) @ W["embed"].T
@@ -186,8 +197,8 @@ def random_weights(cfg, seed, gain=1.0):
         mx = L["mixer"]
         for n in ("norm1", "norm1b"):
             W[p + n] = vec(E)
-        W[p + "mix.q"] = mat(mx["heads"] * mx["dim"], E, 2.0)
-        W[p + "mix.k"] = mat(mx["kv_heads"] * mx["dim"], E, 2.0)
+        W[p + "mix.q"] = mat(mx["heads"] * mx["dim"], E, 1.5)
+        W[p + "mix.k"] = mat(mx["kv_heads"] * mx["dim"], E, 1.5)
         W[p + "mix.v"] = mat(mx["kv_heads"] * mx["vdim"], E)
         W[p + "mix.g"] = mat(mx["heads"] * mx["vdim"], E)
         W[p + "mix.o"] = mat(E, mx["heads"] * mx["vdim"])
