@@ -130,8 +130,99 @@ def rocprof_kernel_us(symbol, args):
         shutil.rmtree(out, ignore_errors=True)
 
 
+# ------------------------------------------------------------------------------------------------ --nigozen: the per-layer model class beside llama
+NIGOZEN_SIZES = {
+    # width, layers, heads, kv heads, head size (keys and values), rotated dims, chunk, dense ff, experts, top, expert ff, vocab
+    "s": dict(width=1024, layers=4, heads=8, kv=2, hd=64, rot=32, chunk=512, ff=4096, experts=8, top=2, eff=1024, vocab=32000),
+    "m": dict(width=2048, layers=4, heads=16, kv=4, hd=128, rot=64, chunk=1024, ff=8192, experts=8, top=2, eff=2048, vocab=32000),
+    "l": dict(width=4096, layers=2, heads=32, kv=8, hd=128, rot=64, chunk=2048, ff=14336, experts=8, top=2, eff=4096, vocab=32000),
+}
+
+
+def nigozen_config(z):
+    """layers alternate a dense and a mixture-of-experts feed-forward; every layer mixes values and is confined to chunks"""
+    layers = []
+    for il in range(z["layers"]):
+        mixer = {"heads": z["heads"], "kv_heads": z["kv"], "dim": z["hd"], "vdim": z["hd"], "mask": {"size": z["chunk"]}, "rot": {"base": 1e6, "dims": z["rot"]},
+                 "scale": z["hd"] ** -0.5, "v_mix": True}
+        mlp = {"kind": "dense", "ff": z["ff"]} if il % 2 == 0 else {"kind": "moe", "expert": {"ff": z["eff"]}, "router": {"experts": z["experts"], "top": z["top"]}}
+        layers.append({"type": "attention", "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Nigozen", "embedding": {"scale": 1.0}, "layers": layers, "norm": {"eps": 1e-5}, "vocab": z["vocab"], "width": z["width"]}
+
+
+def bench_nigozen(args):
+    """Prefill and decode throughput of Nigozen models (bf16 matrices, bf16 cache, random weights) at sizes that resemble real layers, beside the
+    closest existing class at equal size: llama with f16 matrices and an f16 cache (same width, layers, heads, head size, dense ff and vocabulary;
+    its mat-muls run the same mmf.hip tilings on the f16 matrix-core instructions).  One JSON line; per-kernel-class times of both with
+    the bytes each class moved, from the backend's event-bracketed timing (a second, untimed pass)."""
+    import json as _json
+
+    import numpy as np
+
+    import llama_box_amd as L
+    from model_util import Context, Model, preset
+
+    be = L.Backend(0)
+    n_prompt, n_dec, ub = args.prefill, max(8, min(args.steps, 64)), args.ubatch
+    out = {"metric": "nigozen_vs_llama_tokens_per_s", "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16 (nigozen) / f16 (llama)", "data": "synthetic", "prompt": n_prompt,
+           "decode_steps": n_dec, "ubatch": ub, "sizes": {}}
+
+    def run(model, n_vocab):
+        ctx = Context(model, backend=be, n_ctx=n_prompt + n_dec + 256, n_ubatch=ub, flash_attn=1)
+        rng = np.random.default_rng(1)
+        prompt = rng.integers(0, n_vocab, n_prompt).tolist()
+        res = {}
+        for rep in range(2):  # the first pass warms up (graph capture, scratch growth)
+            ctx.clear()
+            be.synchronize()
+            t0 = time.perf_counter()
+            rc, _ = ctx.decode(prompt, range(n_prompt), want=[0] * (n_prompt - 1) + [1], copy_logits=False)
+            assert rc == 0
+            t1 = time.perf_counter()
+            for i in range(n_dec):
+                rc, _ = ctx.decode([prompt[i]], [n_prompt + i], copy_logits=False)
+                assert rc == 0
+            t2 = time.perf_counter()
+            res = {"prefill_tok_s": round(n_prompt / (t1 - t0), 1), "decode_tok_s": round(n_dec / (t2 - t1), 1), "prefill_ms": round((t1 - t0) * 1e3, 2), "decode_ms_per_tok": round((t2 - t1) * 1e3 / n_dec, 3)}
+        # per-class kernel times (eager, event-bracketed): one prompt, a few decode steps
+        be.set_option("timing", 1)
+        ctx.clear()
+        be.timing_report(reset=True)
+        ctx.decode(prompt, range(n_prompt), want=[0] * (n_prompt - 1) + [1], copy_logits=False)
+        pre = be.timing_report(reset=True)
+        for i in range(8):
+            ctx.decode([prompt[i]], [n_prompt + i], copy_logits=False)
+        dec = be.timing_report(reset=True)
+        be.set_option("timing", 0)
+        fmt = lambda rep, div: {k: {"n": v[0] // div, "us": round(v[1] * 1e3 / div, 1), "GB_s": round(v[2] / max(v[1], 1e-9) / 1e6, 1)} for k, v in sorted(rep.items(), key=lambda kv: -kv[1][1]) if v[1] > 0}
+        res["prefill_classes"] = fmt(pre, 1)
+        res["decode_classes"] = fmt(dec, 8)
+        ctx.free()
+        return res
+
+    for name in args.nigozen.split(","):
+        z = NIGOZEN_SIZES[name]
+        cfg = nigozen_config(z)
+        mn = Model(config_json=_json.dumps(cfg), seed=7, buft=be.buft, wtype=L.BF16)
+        r_n = run(mn, z["vocab"])
+        r_n["weight_bytes"] = int(L.host().llm_model_total_bytes(mn.m))
+        r_n["stream_bytes_per_token"] = mn.stream_bytes()
+        mn.free()
+        hp = preset("test-llama", n_layer=z["layers"], n_embd=z["width"], n_head=z["heads"], n_head_kv=z["kv"], n_embd_head=z["hd"], n_ff=z["ff"], n_vocab=z["vocab"], n_ctx_train=8192, ftype=4)
+        ml = Model(hp, 7, be.buft)
+        r_l = run(ml, z["vocab"])
+        r_l["stream_bytes_per_token"] = ml.stream_bytes()
+        ml.free()
+        out["sizes"][name] = {"config": z, "nigozen": r_n, "llama_f16": r_l,
+                              "prefill_ratio": round(r_n["prefill_tok_s"] / r_l["prefill_tok_s"], 3), "decode_ratio": round(r_n["decode_tok_s"] / r_l["decode_tok_s"], 3)}
+    print(_json.dumps(out))
+    be.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--nigozen", default="", help="comma-separated sizes (s, m, l): time prefill and decode of Nigozen models of these sizes beside llama (f16) at equal size, "
+                    "print one JSON line and exit; the default workload is not run")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=8)
@@ -159,6 +250,10 @@ def main():
     ap.add_argument("--timing-steps", type=int, default=16)
     ap.add_argument("--pmc-traffic", type=int, default=1, help="1: re-run a short decode under rocprofv3 --pmc FETCH_SIZE (own pass) for roofline.traffic")
     args = ap.parse_args()
+
+    if args.nigozen:
+        bench_nigozen(args)
+        return
 
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         # `python bench.py --gpus N` on its own: start the N ranks ourselves, exactly as the driver's multi-GPU line does (one process

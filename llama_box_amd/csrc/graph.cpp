@@ -58,8 +58,8 @@ static bool mm_cache_image_ok(const ggml_tensor * op) {
 // which attention path serves this FLASH_ATTN_EXT node: 0 none (the host keeps it on the CPU backend), 1 the f16 kernels on the cache views in place,
 // 2 the lane-parallel kernel on block_q8_0 K / V, 3 the f16 kernels on an f16 IMAGE of whichever of K / V is kept in another type (kv_types.hip:
 // -ctk / -ctv q4_0, q4_1, q5_0, q5_1, iq4_nl, bf16, f32, mixed pairs, and q8_0 shapes route 2 does not take)
-// route 4: the 32-bit kernel over f32 / bf16 / f16 rows read in place (attn_f32.hip) — a cache kept in f32 or bf16 (its values are used as
-// they are, not through an f16 image), head sizes other than 64 / 128, a value size that differs from the key size
+// route 4: the 32-bit kernel over f32 / bf16 / f16 rows read in place (attn_f32.hip) — asked for with an F32 mask (cache values are then used as
+// they are, not through an f16 image), and taken for head sizes other than 64 / 128 or a value size that differs from the key size
 static bool fa_f32_route(const ggml_tensor * op) {
     const ggml_tensor * a = op->src[0];
     const ggml_tensor * k = op->src[1];
@@ -80,7 +80,10 @@ static int fa_route(const ggml_tensor * op) {
         const bool wide_k = k->type == GGML_TYPE_F32 || k->type == GGML_TYPE_BF16, wide_v = v->type == GGML_TYPE_F32 || v->type == GGML_TYPE_BF16;
         const bool plain = (wide_k || k->type == GGML_TYPE_F16) && (wide_v || v->type == GGML_TYPE_F16);
         const bool odd_shape = k->ne[0] != v->ne[0] || (k->ne[0] != 64 && k->ne[0] != 128);
-        if (plain && ((wide_k && wide_v) || odd_shape) && fa_f32_route(op)) return 4;
+        // an F32 mask (not the F16 cast flash attention is usually handed) is how a graph asks for the 32-bit kernel at shapes the f16 kernels serve too
+        const bool f32_mask = m && m->type == GGML_TYPE_F32;
+        (void) wide_k; (void) wide_v;
+        if (plain && (f32_mask || odd_shape) && fa_f32_route(op)) return 4;
     }
     if (k->type == GGML_TYPE_Q8_0 && v->type == GGML_TYPE_Q8_0) {
         // quantised KV cache: served by the lane-parallel kernel (head_dim 128, 1 .. 8 query heads per KV head, no soft-capping / ALiBi)
@@ -1691,6 +1694,52 @@ static bool try_fuse_attn_nf_mma(exec_state & st, int i) {
     return true;
 }
 
+// MUL(rows [n, n_used, T], w [1, n_used, T]) followed by the sum over the used experts written as views of the product and a chain of ADDs (one used
+// expert: a CONT of the one view): a single pass that writes the chain's last node.  Returns the number of nodes consumed (0: not that pattern).
+static int try_fuse_expert_sum(exec_state & st, int i) {
+    backend_ctx * c = st.c;
+    ggml_cgraph * g = st.g;
+    const ggml_tensor * mul = g->nodes[i];
+    const ggml_tensor * rows = mul->src[0], * w = mul->src[1];
+    if (!rows || !w || rows->op != GGML_OP_MUL_MAT_ID || !is_f32_contig(rows) || !is_f32_contig(mul) || w->type != GGML_TYPE_F32 || w->nb[0] != 4) return 0;
+    const int64_t n = rows->ne[0], n_used = rows->ne[1], T = rows->ne[2];
+    if (rows->ne[3] != 1 || w->ne[0] != 1 || w->ne[1] != n_used || w->ne[2] != T || w->ne[3] != 1 || !same_shape(mul, rows) || (mul->flags & GGML_TENSOR_FLAG_OUTPUT)) return 0;
+    // the chain: view 0, view 1, ADD, view 2, ADD, ... in the graph's order, every link read once
+    int k = i + 1, views = 0;
+    const ggml_tensor * acc = nullptr;
+    auto is_slice = [&](const ggml_tensor * t, int64_t u) {
+        return t->op == GGML_OP_VIEW && t->view_src == mul && t->ne[0] == n && t->ne[1] == T && t->ne[2] == 1 && t->ne[3] == 1 && t->nb[1] == mul->nb[2] && t->view_offs == (size_t) u * mul->nb[1];
+    };
+    for (; k < g->n_nodes && views < n_used; ++k) {
+        const ggml_tensor * t = g->nodes[k];
+        if (st.done[k]) return 0;
+        if (is_slice(t, views)) {
+            if (views == 0) { acc = t; ++views; continue; }
+            const ggml_tensor * ad = k + 1 < g->n_nodes ? g->nodes[k + 1] : nullptr;
+            if (!ad || st.done[k + 1] || ad->op != GGML_OP_ADD || ad->src[0] != acc || ad->src[1] != t || !is_f32_contig(ad) || ad->ne[0] != n || ad->ne[1] != T) return 0;
+            if (views + 1 < n_used && ((ad->flags & GGML_TENSOR_FLAG_OUTPUT) || !single_use(st, ad))) return 0;
+            acc = ad;
+            ++views;
+            ++k;
+            continue;
+        }
+        return 0;
+    }
+    if (views != n_used || !acc) return 0;
+    if (n_used == 1) {  // the one slice is made contiguous by a CONT
+        const ggml_tensor * ct = k < g->n_nodes ? g->nodes[k] : nullptr;
+        if (!ct || st.done[k] || ct->op != GGML_OP_CONT || ct->src[0] != acc || !is_f32_contig(ct)) return 0;
+        acc = ct;
+        ++k;
+    }
+    if (use_count(st, mul) != (int) n_used) return 0;  // nothing else reads the product
+    if (ranges_overlap(acc, rows) || ranges_overlap(acc, w)) return 0;
+    launch_weighted_rows_sum(c->stream, TD(rows), TD(w), TD(acc));
+    c->st.kernel_launches++;
+    c->st.fused_nodes += k - i - 1;
+    return k - i;
+}
+
 static int run_node(exec_state & st, int i) {
     backend_ctx * c = st.c;
     ggml_cgraph * g = st.g;
@@ -1900,16 +1949,42 @@ static int run_node(exec_state & st, int i) {
         }
 
         case GGML_OP_ADD: case GGML_OP_SUB: case GGML_OP_MUL: case GGML_OP_DIV: {
+            if (fuse && n->op == GGML_OP_MUL) {
+                const int used = try_fuse_expert_sum(st, i);
+                if (used > 0) return used;
+            }
             timed_scope ts(c, "binary", (double) ggml_abi_nbytes(n) * 3);
             launch_binary(s, n->op, TD(a), TD(b), TD(n));
             c->st.kernel_launches++;
             return 1;
         }
-        case GGML_OP_SCALE:
+        case GGML_OP_SCALE: {
+            // SCALE(x, a), SCALE(y, b), ADD of the two (a blend of two tensors): one pass
+            ggml_tensor * s2 = next(1), * ad = next(2);
+            if (fuse && s2 && ad && s2->op == GGML_OP_SCALE && ad->op == GGML_OP_ADD && ((ad->src[0] == n && ad->src[1] == s2) || (ad->src[0] == s2 && ad->src[1] == n)) &&
+                ggml_abi_op_param_f32(n, 1) == 0.0f && ggml_abi_op_param_f32(s2, 1) == 0.0f && single_use(st, n) && single_use(st, s2) && is_f32_contig(s2->src[0]) && is_f32_contig(ad) &&
+                same_shape(n, s2) && same_shape(n, ad) && !(ranges_overlap(ad, a) && ad->data != a->data) && !(ranges_overlap(ad, s2->src[0]) && ad->data != s2->src[0]->data)) {
+                launch_axpby(s, (const float *) a->data, ggml_abi_op_param_f32(n, 0), (const float *) s2->src[0]->data, ggml_abi_op_param_f32(s2, 0), (float *) ad->data, ggml_abi_nelements(ad));
+                c->st.kernel_launches++;
+                c->st.fused_nodes += 2;
+                return 3;
+            }
             launch_scale(s, TD(a), TD(n), ggml_abi_op_param_f32(n, 0), ggml_abi_op_param_f32(n, 1));
             c->st.kernel_launches++;
             return 1;
+        }
         case GGML_OP_UNARY: {
+            // SIGMOID(g) -> MUL(x, sigmoid): a gate in one pass
+            ggml_tensor * gm = next(1);
+            if (fuse && n->op_params[0] == GGML_UNARY_OP_SIGMOID && gm && gm->op == GGML_OP_MUL && (gm->src[0] == n || gm->src[1] == n) && gm->src[0] != gm->src[1] && single_use(st, n)) {
+                const ggml_tensor * x = gm->src[0] == n ? gm->src[1] : gm->src[0];
+                if (is_f32_contig(x) && is_f32_contig(gm) && same_shape(x, n) && same_shape(gm, n)) {
+                    launch_mul_sigmoid(s, (const float *) x->data, (const float *) a->data, (float *) gm->data, ggml_abi_nelements(gm));
+                    c->st.kernel_launches++;
+                    c->st.fused_nodes++;
+                    return 2;
+                }
+            }
             // RELU -> SQR (the squared-ReLU activation): one pass writing the SQR's output
             ggml_tensor * sq = next(1);
             if (fuse && n->op_params[0] == GGML_UNARY_OP_RELU && sq && sq->op == GGML_OP_SQR && sq->src[0] == n && single_use(st, n) && is_f32_contig(sq) && same_shape(sq, n)) {

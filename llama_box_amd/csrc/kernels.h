@@ -229,6 +229,9 @@ void launch_argsort(hipStream_t s, const tdesc & src, const tdesc & dst, int des
 // element-wise forms outside ggml's unary enumeration, served by launch_unary: x^2 (SQR) and relu(x)^2 (RELU followed by SQR)
 #define MI_UNARY_SQR 1000
 #define MI_UNARY_RELU_SQR 1001
+void launch_axpby(hipStream_t s, const float * x, float a, const float * y, float b, float * d, int64_t n);  // d = a x + b y (each product rounded, then the sum: SCALE, SCALE, ADD)
+void launch_mul_sigmoid(hipStream_t s, const float * x, const float * g, float * d, int64_t n);          // d = x * sigmoid(g)
+void launch_weighted_rows_sum(hipStream_t s, const tdesc & rows /* [n, n_used, T] */, const tdesc & w /* [1, n_used, T] */, const tdesc & d /* [n, T] */);
 void launch_binary(hipStream_t s, int op, const tdesc & a, const tdesc & b, const tdesc & dst);
 void launch_scale(hipStream_t s, const tdesc & src, const tdesc & dst, float scale, float bias);
 void launch_unary(hipStream_t s, int uop, const tdesc & src, const tdesc & dst);

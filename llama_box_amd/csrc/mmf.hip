@@ -368,20 +368,20 @@ size_t mul_mat_f_workspace_bytes(const tdesc & a, const tdesc & b) {
 //   long rows (V^T.p: K = cells): a wave owns 4 rows, the 4 waves of the workgroup take K in interleaved 512-element slices and
 //   add up through LDS.
 // f32 accumulation in a different order than the dot kernel (and the CPU); same NMSE gate (tests/test_gpu_ops.py::test_mul_mat_f).
-__device__ __forceinline__ void mmf_w8(const char * p, float (&w)[8]) {
+template <bool BF = false> __device__ __forceinline__ void mmf_w8(const char * p, float (&w)[8]) {
     const uint4 t = *(const uint4 *) p;
     const uint32_t u[4] = {t.x, t.y, t.z, t.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        w[2 * i] = h2f((uint16_t) (u[i] & 0xFFFF));
-        w[2 * i + 1] = h2f((uint16_t) (u[i] >> 16));
+        w[2 * i] = BF ? __uint_as_float(u[i] << 16) : h2f((uint16_t) (u[i] & 0xFFFF));
+        w[2 * i + 1] = BF ? __uint_as_float(u[i] & 0xFFFF0000u) : h2f((uint16_t) (u[i] >> 16));
     }
 }
-__device__ __forceinline__ void mmf_x8(const char * p, float (&x)[8]) {
+template <bool BF = false> __device__ __forceinline__ void mmf_x8(const char * p, float (&x)[8]) {
     const float4 x0 = *(const float4 *) p, x1 = *(const float4 *) (p + 16);
     const float t[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
 #pragma unroll
-    for (int i = 0; i < 8; ++i) x[i] = h2f(f2h(t[i]));
+    for (int i = 0; i < 8; ++i) x[i] = BF ? mmf_bf16_round(t[i]) : h2f(f2h(t[i]));
 }
 // sum over each group of LPR consecutive lanes, on the DPP path (the 64 ds_bpermute a shuffle butterfly needs here — 16 sums, 4
 // dependent steps each — were 3.7 of the kernel's 7.8 us: scripts/ubench/attn_probe.hip)
@@ -397,7 +397,7 @@ template <int LPR> __device__ __forceinline__ float group_sum(float v) {
     v += dpp_f32<MI_DPP_HALF_MIRROR>(v);
     return v;
 }
-template <int G, int LPR>
+template <int G, int LPR, bool BF = false>
 __global__ void __launch_bounds__(256) k_mul_mat_f16_gqa_short(const tdesc a, const tdesc b, const tdesc d) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     constexpr int lpr = LPR;
@@ -408,7 +408,7 @@ __global__ void __launch_bounds__(256) k_mul_mat_f16_gqa_short(const tdesc a, co
     float x[G][8];
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-        if (kin) mmf_x8(b.data + (i02 * G + g) * b.nb[2] + (int64_t) sl * 32, x[g]);
+        if (kin) mmf_x8<BF>(b.data + (i02 * G + g) * b.nb[2] + (int64_t) sl * 32, x[g]);
         else
 #pragma unroll
             for (int i = 0; i < 8; ++i) x[g][i] = 0.0f;
@@ -417,7 +417,7 @@ __global__ void __launch_bounds__(256) k_mul_mat_f16_gqa_short(const tdesc a, co
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int64_t row = std::min<int64_t>(base + 4 * rpw * r, a.ne[1] - 1);
-        if (kin) mmf_w8(a.data + row * a.nb[1] + i02 * a.nb[2] + (int64_t) sl * 16, w[r]);
+        if (kin) mmf_w8<BF>(a.data + row * a.nb[1] + i02 * a.nb[2] + (int64_t) sl * 16, w[r]);
         else
 #pragma unroll
             for (int i = 0; i < 8; ++i) w[r][i] = 0.0f;
@@ -435,7 +435,7 @@ __global__ void __launch_bounds__(256) k_mul_mat_f16_gqa_short(const tdesc a, co
         }
     }
 }
-template <int G>
+template <int G, bool BF = false>
 __global__ void __launch_bounds__(256) k_mul_mat_f16_gqa_long(const tdesc a, const tdesc b, const tdesc d) {
     __shared__ float part[4][4 * G];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -451,10 +451,10 @@ __global__ void __launch_bounds__(256) k_mul_mat_f16_gqa_long(const tdesc a, con
     for (int64_t k = (int64_t) wave * 512 + lane * 8; k < K; k += 2048) {
         float w[4][8], x[8];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) mmf_w8(wr[r] + k * 2, w[r]);
+        for (int r = 0; r < 4; ++r) mmf_w8<BF>(wr[r] + k * 2, w[r]);
 #pragma unroll
         for (int g = 0; g < G; ++g) {
-            mmf_x8(b.data + (i02 * G + g) * b.nb[2] + k * 4, x);
+            mmf_x8<BF>(b.data + (i02 * G + g) * b.nb[2] + k * 4, x);
 #pragma unroll
             for (int r = 0; r < 4; ++r)
 #pragma unroll
@@ -706,6 +706,25 @@ bool launch_soft_max_mul_mat_f16(hipStream_t s, const tdesc & a, const tdesc & k
     return false;
 }
 
+// one column against a bf16 matrix (a decode step's projections): the same two forms on bf16 rows
+static void launch_matvec_bf16(hipStream_t s, const tdesc & a, const tdesc & b, const tdesc & d) {
+    const int64_t K = a.ne[0];
+    if (K <= 512) {
+        int lpr = 64;
+        while (lpr > 8 && (int64_t) (lpr / 2) * 8 >= K) lpr >>= 1;
+        const int rows_per_block = 16 * (64 / lpr);
+        dim3 grid((unsigned) ((a.ne[1] + rows_per_block - 1) / rows_per_block), (unsigned) a.ne[2]);
+        switch (lpr) {
+            case 8: hipLaunchKernelGGL((k_mul_mat_f16_gqa_short<1, 8, true>), grid, dim3(256), 0, s, a, b, d); break;
+            case 16: hipLaunchKernelGGL((k_mul_mat_f16_gqa_short<1, 16, true>), grid, dim3(256), 0, s, a, b, d); break;
+            case 32: hipLaunchKernelGGL((k_mul_mat_f16_gqa_short<1, 32, true>), grid, dim3(256), 0, s, a, b, d); break;
+            default: hipLaunchKernelGGL((k_mul_mat_f16_gqa_short<1, 64, true>), grid, dim3(256), 0, s, a, b, d); break;
+        }
+    } else {
+        dim3 grid((unsigned) ((a.ne[1] + 3) / 4), (unsigned) a.ne[2]);
+        hipLaunchKernelGGL((k_mul_mat_f16_gqa_long<1, true>), grid, dim3(256), 0, s, a, b, d);
+    }
+}
 template <int G> static void launch_gqa_t(hipStream_t s, const tdesc & a, const tdesc & b, const tdesc & d) {
     const int64_t K = a.ne[0];
     if (K <= 512) {
@@ -768,6 +787,10 @@ void launch_mul_mat_f(hipStream_t s, const tdesc & a, const tdesc & b, const tde
         dim3 grid((unsigned) ((a.ne[1] + 63) / 64), (unsigned) ((b.ne[1] + 63) / 64), (unsigned) (b.ne[2] * b.ne[3]));
         if (bf) hipLaunchKernelGGL(k_mul_mat_f16_mma<true>, grid, dim3(256), 0, s, a, b, d);
         else hipLaunchKernelGGL(k_mul_mat_f16_mma<false>, grid, dim3(256), 0, s, a, b, d);
+        return;
+    }
+    if (bf && vec_ok && b.ne[1] == 1 && a.ne[3] == 1 && b.ne[3] == 1 && b.ne[2] == a.ne[2] && a.ne[1] >= 64) {
+        launch_matvec_bf16(s, a, b, d);
         return;
     }
     if (w16 && !bf && vec_ok && b.ne[1] == 1 && a.ne[3] == 1 && b.ne[3] == 1 && b.ne[2] % a.ne[2] == 0 && a.ne[1] >= 64) {  // a decode step's K.q / V^T.p

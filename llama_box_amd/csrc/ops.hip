@@ -196,6 +196,47 @@ void launch_argsort(hipStream_t s, const tdesc & src, const tdesc & dst, int des
     hipLaunchKernelGGL(k_argsort, dim3((unsigned) rows), dim3(256), 0, s, src, dst, descending);
 }
 
+// ------------------------------------------------------------------------------------------------ small fused element-wise forms
+// a x + b y (two SCALEs and the ADD of a blend), x * sigmoid(g) (a gate), and the weighted sum over the used experts of a mixture-of-experts
+// block: dst[:, t] = sum_u w[u, t] * rows[:, u, t] (the MUL by the router weights and the ADD chain over views, in the chain's order)
+__global__ void __launch_bounds__(256) k_axpby(const float * __restrict__ x, const float a, const float * __restrict__ y, const float b, float * __restrict__ d, const int64_t n) {
+    for (int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t) gridDim.x * blockDim.x) {
+        const float p = x[i] * a, q = y[i] * b;
+        d[i] = p + q;
+    }
+}
+void launch_axpby(hipStream_t s, const float * x, float a, const float * y, float b, float * d, int64_t n) {
+    if (n == 0) return;
+    hipLaunchKernelGGL(k_axpby, dim3((unsigned) std::min<int64_t>((n + 255) / 256, 2048)), dim3(256), 0, s, x, a, y, b, d, n);
+}
+__global__ void __launch_bounds__(256) k_mul_sigmoid(const float * __restrict__ x, const float * __restrict__ g, float * __restrict__ d, const int64_t n) {
+    for (int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t) gridDim.x * blockDim.x) {
+        const float sg = 1.f / (1.f + expf(-g[i]));
+        d[i] = x[i] * sg;
+    }
+}
+void launch_mul_sigmoid(hipStream_t s, const float * x, const float * g, float * d, int64_t n) {
+    if (n == 0) return;
+    hipLaunchKernelGGL(k_mul_sigmoid, dim3((unsigned) std::min<int64_t>((n + 255) / 256, 2048)), dim3(256), 0, s, x, g, d, n);
+}
+__global__ void __launch_bounds__(256) k_weighted_rows_sum(const tdesc rows, const tdesc w, const tdesc d) {
+    const int64_t t = blockIdx.x, n_used = rows.ne[1];
+    const float * __restrict__ wt = (const float *) (w.data + t * w.nb[2]);
+    float * __restrict__ out = (float *) (d.data + t * d.nb[1]);
+    for (int64_t i = threadIdx.x; i < rows.ne[0]; i += blockDim.x) {
+        float acc = 0.0f;
+        for (int64_t u = 0; u < n_used; ++u) {
+            const float p = *(const float *) (rows.data + i * 4 + u * rows.nb[1] + t * rows.nb[2]) * *(const float *) ((const char *) wt + u * w.nb[1]);
+            acc = u == 0 ? p : acc + p;
+        }
+        out[i] = acc;
+    }
+}
+void launch_weighted_rows_sum(hipStream_t s, const tdesc & rows, const tdesc & w, const tdesc & d) {
+    if (rows.ne[2] == 0) return;
+    hipLaunchKernelGGL(k_weighted_rows_sum, dim3((unsigned) rows.ne[2]), dim3(256), 0, s, rows, w, d);
+}
+
 // ------------------------------------------------------------------------------------------------ ADD/SUB/MUL/DIV
 __global__ void __launch_bounds__(256) k_binary(const int op, const tdesc a, const tdesc b, const tdesc d) {
     const int64_t row = blockIdx.x;

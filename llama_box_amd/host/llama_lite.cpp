@@ -1289,8 +1289,8 @@ static void build_layerwise(llm_context * c, ggml_context * ctx, ggml_cgraph * g
     llm_model * m = c->model;
     const llm_hparams & hp = m->hp;
     const float eps = hp.rms_eps;
-    std::vector<ggml_tensor *> mask_cnv;
-    for (size_t k = 0; k < io.masks.size(); ++k) mask_cnv.push_back(named(ggml_cast(ctx, io.masks[k], GGML_TYPE_F16), "KQ_mask_cnv", (int) k));
+    // the F32 masks go to FLASH_ATTN_EXT as they are (no F16 cast): that is how this graph asks the backend for attention in 32-bit arithmetic
+    const std::vector<ggml_tensor *> & mask_cnv = io.masks;
     ggml_tensor * inpL = named(ggml_get_rows(ctx, m->tok_embd, io.tokens), "inp_embd", -1);
     if (m->embd_scale != 1.0f) inpL = named(ggml_scale(ctx, inpL, m->embd_scale), "inp_scaled", -1);
     ggml_tensor * v_first = nullptr;

@@ -221,7 +221,7 @@ def attention_case(backend, H, kv_type, n_q, n_kv, heads, kv_heads, dk, dv, chun
         esz = 2 if kv_type == L.BF16 else 4
         kk = H.ggml_view_3d(g.ctx, tk, dk, n_kv, kv_heads, dk * kv_heads * esz, dk * esz, 0)
         vv = H.ggml_view_3d(g.ctx, tv, dv, n_kv, kv_heads, dv * kv_heads * esz, dv * esz, 0)
-        r = H.ggml_flash_attn_ext(g.ctx, H.ggml_permute(g.ctx, tq, 0, 2, 1, 3), kk, vv, g.new(L.F16, [n_kv, mask.shape[0]], mask.astype(np.float16)), 0.25, 0.0, 0.0)
+        r = H.ggml_flash_attn_ext(g.ctx, H.ggml_permute(g.ctx, tq, 0, 2, 1, 3), kk, vv, g.new(L.F32, [n_kv, mask.shape[0]], mask), 0.25, 0.0, 0.0)  # an F32 mask: the 32-bit kernel
         H.ggml_flash_attn_ext_set_prec(r, 10)
         if sink:
             H.ggml_flash_attn_ext_add_sinks(r, g.new(L.F32, [heads], np.zeros(heads, np.float32)))

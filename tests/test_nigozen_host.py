@@ -76,7 +76,7 @@ def _graph_probe(H, m, n_ctx, steps):
             name = H.ggml_op_name(t.op).decode()
             ops[name] = ops.get(name, 0) + 1
             for s in range(4):
-                if t.src[s] and t.src[s].contents.name.startswith(b"KQ_mask") and b"cnv" not in t.src[s].contents.name:
+                if t.src[s] and t.src[s].contents.name.startswith(b"KQ_mask"):
                     mt = t.src[s].contents
                     arr = np.ctypeslib.as_array(C.cast(mt.data, C.POINTER(C.c_float)), shape=(mt.ne[1], mt.ne[0])).copy()
                     masks[mt.name.decode()] = arr
