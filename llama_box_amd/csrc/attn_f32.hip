@@ -12,6 +12,7 @@
 //                      f32 once per workgroup and every wave runs 16 of the queries against them (a lane owns one cell for the scores
 //                      and one or more value columns for the sum); blocks the mask hides from all 64 queries are skipped.
 #include <algorithm>
+#include <cstdlib>
 
 #include "dev_util.h"
 #include "kernels.h"
@@ -220,6 +221,169 @@ __global__ void __launch_bounds__(256) k_attn_f32_tile(const tdesc q, const tdes
     }
 }
 
+// ------------------------------------------------------------------------------------------------ prompt batches over a bf16 cache: the matrix cores
+// k_attn_mma_bf16: a workgroup owns 128 query tokens of one head, a wave 32 of them.  Per block of 32 cells
+//   S^T = K . Q^T   on v_mfma_f32_32x32x16_bf16 (first operand: the cells' bf16 rows straight from the cache, 16 bytes a lane; second: the wave's queries,
+//                   rounded to bf16 once and kept in registers) — a lane then holds 16 scores of ITS query (its half-wave's cells), so the running maximum,
+//                   the sum and the rescaling are per-lane scalars and one exchange with the other half-wave;
+//   scores, maxima, exponentials and sums are f32;
+//   O^T += V^T . P^T  on the same instruction, V^T staged through LDS (bf16, transposed on the way in), the weights P given as TWO bf16 terms
+//                   (p = hi + lo, |lo| <= 2^-9 |p|): the f32 weights enter the sum to 2^-17, not rounded to 8 bits.
+// The key order inside the second product is the order the first product's registers come in (both operands permuted alike).
+// Blocks that the mask hides from all 128 queries are skipped after the mask read.  Head sizes: multiples of 8 up to 16 DK16 / 32 DVT.
+typedef __bf16 att_bf8 __attribute__((ext_vector_type(8)));
+typedef float att_f16v __attribute__((ext_vector_type(16)));
+__device__ __forceinline__ uint32_t att_bf16_bits(const float f) {
+    const uint32_t u = __float_as_uint(f);
+    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+template <int DK16, int DVT>
+__global__ void __launch_bounds__(256) k_attn_mma_bf16(const tdesc q, const tdesc k, const tdesc v, const tdesc mask, const float * __restrict__ sinks, const tdesc dst, const float scale) {
+    constexpr int VS = 36;  // V^T row stride in LDS (bf16 elements): 72 bytes keeps the 8-byte reads aligned and spreads the rows over the banks
+    __shared__ uint16_t Vt[DVT * 32 * VS];
+    __shared__ int flag[2];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n = lane & 31, g = lane >> 5;
+    const int64_t h = blockIdx.y, n_q = q.ne[1], n_kv = k.ne[1];
+    const int DK = (int) q.ne[0], DV = (int) v.ne[0];
+    const int64_t tq = (int64_t) blockIdx.x * 128 + wave * 32 + n;  // this lane's query
+    const bool q_live = tq < n_q;
+    const int64_t kvh = h / (q.ne[2] / k.ne[2]);
+    const char * kbase = k.data + kvh * k.nb[2];
+    const char * vbase = v.data + kvh * v.nb[2];
+    // the wave's queries as second operands: element group (16 s + 8 g .. + 7) of query n
+    uint4 qf[DK16];
+    {
+        const float * qrow = (const float *) (q.data + (q_live ? tq : 0) * q.nb[1] + h * q.nb[2]);
+#pragma unroll
+        for (int s = 0; s < DK16; ++s) {
+            const int i0 = 16 * s + 8 * g;
+            uint32_t b[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) b[e] = (q_live && i0 + e < DK) ? att_bf16_bits(qrow[i0 + e]) : 0u;
+            qf[s] = make_uint4(b[0] | (b[1] << 16), b[2] | (b[3] << 16), b[4] | (b[5] << 16), b[6] | (b[7] << 16));
+        }
+    }
+    float m = sinks ? sinks[h] : ATTN_F32_LOW, l = sinks ? 1.0f : 0.0f;
+    att_f16v O[DVT];
+#pragma unroll
+    for (int dt = 0; dt < DVT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) O[dt][i] = 0.0f;
+    const char * mrow = mask.data + (q_live ? tq : 0) * mask.nb[1];
+    if (threadIdx.x < 2) flag[threadIdx.x] = 0;
+    __syncthreads();
+    for (int64_t j0 = 0, blk = 0; j0 < n_kv; j0 += 32, ++blk) {
+        // this lane's 16 mask terms: cells j0 + 8 b + 4 g .. + 3, b = 0 .. 3 (register i = 4 b + r)
+        float mv[16];
+        bool any = false;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int64_t j = j0 + 8 * b + 4 * g;
+            float4 t = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+            if (q_live && j + 3 < n_kv) t = *(const float4 *) (mrow + j * 4);
+            else if (q_live) {
+                if (j < n_kv) t.x = ((const float *) mrow)[j];
+                if (j + 1 < n_kv) t.y = ((const float *) mrow)[j + 1];
+                if (j + 2 < n_kv) t.z = ((const float *) mrow)[j + 2];
+            }
+            mv[4 * b] = t.x; mv[4 * b + 1] = t.y; mv[4 * b + 2] = t.z; mv[4 * b + 3] = t.w;
+            any = any || t.x > -INFINITY || t.y > -INFINITY || t.z > -INFINITY || t.w > -INFINITY;
+        }
+        const bool wave_any = __ballot(any) != 0;
+        if (threadIdx.x == 0) flag[(blk + 1) & 1] = 0;
+        if (wave_any && lane == 0) flag[blk & 1] = 1;
+        __syncthreads();
+        if (!flag[blk & 1]) continue;  // (the same answer for every thread of the workgroup)
+        // V^T of the block into LDS: thread takes 8 consecutive value entries of one cell
+        for (int e0 = threadIdx.x; e0 < 32 * (DVT * 4); e0 += 256) {
+            const int cell = e0 / (DVT * 4), c8 = e0 % (DVT * 4);
+            uint4 t = make_uint4(0, 0, 0, 0);
+            if (j0 + cell < n_kv && 8 * c8 < DV) t = *(const uint4 *) (vbase + (j0 + cell) * v.nb[1] + c8 * 16);
+            const uint32_t u[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                Vt[(8 * c8 + 2 * e) * VS + cell] = (uint16_t) (u[e] & 0xFFFF);
+                Vt[(8 * c8 + 2 * e + 1) * VS + cell] = (uint16_t) (u[e] >> 16);
+            }
+        }
+        __syncthreads();
+        if (!wave_any) continue;  // (wave-uniform; no barrier follows inside this iteration)
+        att_f16v S;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) S[i] = 0.0f;
+        {
+            const int64_t cell = j0 + n < n_kv ? j0 + n : n_kv - 1;
+            const char * krow = kbase + cell * k.nb[1] + g * 16;
+#pragma unroll
+            for (int s = 0; s < DK16; ++s) {
+                uint4 kf = make_uint4(0, 0, 0, 0);
+                if (16 * s + 8 * g < DK) kf = *(const uint4 *) (krow + s * 32);
+                S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(att_bf8, kf), __builtin_bit_cast(att_bf8, qf[s]), S, 0, 0, 0);
+            }
+        }
+        float mx = ATTN_F32_LOW;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            S[i] = mv[i] > -INFINITY ? S[i] * scale + mv[i] : -INFINITY;
+            mx = fmaxf(mx, S[i]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m, mx);
+        const float corr = expf(m - m_new);
+        float ps = 0.0f;
+        uint32_t hi[8], lo[8];
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) {
+            const float p0 = expf(S[i] - m_new), p1 = expf(S[i + 1] - m_new);
+            ps += p0 + p1;
+            const uint32_t h0 = att_bf16_bits(p0), h1 = att_bf16_bits(p1);
+            hi[i >> 1] = h0 | (h1 << 16);
+            lo[i >> 1] = att_bf16_bits(p0 - __uint_as_float(h0 << 16)) | (att_bf16_bits(p1 - __uint_as_float(h1 << 16)) << 16);
+        }
+        ps += __shfl_xor(ps, 32, 64);
+        l = l * corr + ps;
+        m = m_new;
+#pragma unroll
+        for (int dt = 0; dt < DVT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) O[dt][i] *= corr;
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            const uint4 ph = make_uint4(hi[4 * s2], hi[4 * s2 + 1], hi[4 * s2 + 2], hi[4 * s2 + 3]);
+            const uint4 pl = make_uint4(lo[4 * s2], lo[4 * s2 + 1], lo[4 * s2 + 2], lo[4 * s2 + 3]);
+#pragma unroll
+            for (int dt = 0; dt < DVT; ++dt) {
+                const uint16_t * vr = Vt + (32 * dt + n) * VS + 16 * s2 + 4 * g;
+                const uint2 a0 = *(const uint2 *) vr, a1 = *(const uint2 *) (vr + 8);
+                const uint4 vf = make_uint4(a0.x, a0.y, a1.x, a1.y);
+                O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(att_bf8, vf), __builtin_bit_cast(att_bf8, ph), O[dt], 0, 0, 0);
+                O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(att_bf8, vf), __builtin_bit_cast(att_bf8, pl), O[dt], 0, 0, 0);
+            }
+        }
+    }
+    if (!q_live) return;
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    float * out = (float *) (dst.data + h * dst.nb[1] + tq * dst.nb[2]);
+#pragma unroll
+    for (int dt = 0; dt < DVT; ++dt)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int d0 = 32 * dt + 8 * b + 4 * g;
+            if (d0 + 3 < DV) *(float4 *) (out + d0) = make_float4(O[dt][4 * b] * inv, O[dt][4 * b + 1] * inv, O[dt][4 * b + 2] * inv, O[dt][4 * b + 3] * inv);
+            else
+                for (int r = 0; r < 4; ++r) if (d0 + r < DV) out[d0 + r] = O[dt][4 * b + r] * inv;
+        }
+}
+static bool attn_mma_bf16_ok(const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const tdesc & dst) {
+    if (!mask || mask->type != GGML_TYPE_F32 || (mask->nb[1] % 16) != 0 || (((uintptr_t) mask->data) & 15)) return false;
+    if (k.type != GGML_TYPE_BF16 || v.type != GGML_TYPE_BF16 || q.ne[1] < 32) return false;
+    if ((q.ne[0] % 8) != 0 || (v.ne[0] % 8) != 0 || q.ne[0] > 128 || v.ne[0] > 128) return false;
+    if ((k.nb[1] % 16) || (k.nb[2] % 16) || (v.nb[1] % 16) || (v.nb[2] % 16) || (((uintptr_t) k.data | (uintptr_t) v.data | (uintptr_t) dst.data) & 15)) return false;
+    if ((dst.nb[1] % 16) || (dst.nb[2] % 16)) return false;
+    return true;
+}
+
 static bool attn_f32_type_ok(int t) { return t == GGML_TYPE_F32 || t == GGML_TYPE_BF16 || t == GGML_TYPE_F16; }
 
 // may launch_attn_f32 serve this op?  q f32 [DK, n_q, H], k [DK, n_kv, G], v [DV, n_kv, G] of one type each, rows contiguous, one batch
@@ -238,6 +402,20 @@ template <int KT, int VT>
 static void attn_f32_launch_t(hipStream_t s, const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const float * sinks, const tdesc & dst, float scale) {
     const int64_t n_q = q.ne[1], H = q.ne[2];
     const int DK = (int) q.ne[0], DV = (int) v.ne[0];
+    if constexpr (KT == GGML_TYPE_BF16 && VT == GGML_TYPE_BF16) {
+        static const bool mma_on = !getenv("GGML_MI355X_ATTN_MMA") || atoi(getenv("GGML_MI355X_ATTN_MMA")) != 0;
+        if (mma_on && attn_mma_bf16_ok(q, k, v, mask, dst)) {  // prompt portions over a bf16 cache: the matrix cores
+            const dim3 grid((unsigned) ((n_q + 127) / 128), (unsigned) H);
+            const int dk16 = (DK + 15) / 16, dvt = (DV + 31) / 32;
+#define MI_ATT_MMA(A, B) hipLaunchKernelGGL((k_attn_mma_bf16<A, B>), grid, dim3(256), 0, s, q, k, v, *mask, sinks, dst, scale)
+            const int a = dk16 <= 2 ? 2 : (dk16 <= 4 ? 4 : 8), b = dvt <= 1 ? 1 : (dvt <= 2 ? 2 : 4);
+            if (a == 2 && b == 1) MI_ATT_MMA(2, 1); else if (a == 2 && b == 2) MI_ATT_MMA(2, 2); else if (a == 2) MI_ATT_MMA(2, 4);
+            else if (a == 4 && b == 1) MI_ATT_MMA(4, 1); else if (a == 4 && b == 2) MI_ATT_MMA(4, 2); else if (a == 4) MI_ATT_MMA(4, 4);
+            else if (b == 1) MI_ATT_MMA(8, 1); else if (b == 2) MI_ATT_MMA(8, 2); else MI_ATT_MMA(8, 4);
+#undef MI_ATT_MMA
+            return;
+        }
+    }
     // the tile kernel: batches of 32 queries and more under a mask, head sizes up to 128 (its LDS: 64 cells of K and V plus 64 queries as f32)
     if (mask && n_q >= 32 && DK <= 128 && DV <= 128) {
         const dim3 grid((unsigned) ((n_q + 63) / 64), (unsigned) H);

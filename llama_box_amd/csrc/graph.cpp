@@ -1694,6 +1694,58 @@ static bool try_fuse_attn_nf_mma(exec_state & st, int i) {
     return true;
 }
 
+// A decode step's bf16 projections of the same activations (q, k, v and the gate of a layer): the siblings that follow node i are executed EARLY, at node i,
+// as one launch — legal when nothing between node i and a sibling's own position reads or occupies the memory the sibling's result goes to (the graph
+// allocator may have given it a block that an earlier tensor still owns at node i's time).  Returns true when node i and at least one sibling were served.
+static bool try_merge_matvec_bf16(exec_state & st, int i) {
+    backend_ctx * c = st.c;
+    ggml_cgraph * g = st.g;
+    const ggml_tensor * n0 = g->nodes[i];
+    const ggml_tensor * X = n0->src[1];
+    const int64_t K = n0->src[0]->ne[0];
+    if (!is_f32_contig(X) || ggml_abi_nelements(X) != K || (K % 8) != 0 || K < 256 || (((uintptr_t) X->data) & 15)) return false;
+    auto eligible = [&](const ggml_tensor * t) {
+        const ggml_tensor * w = t->src[0];
+        return t->op == GGML_OP_MUL_MAT && t->src[1] == X && w->type == GGML_TYPE_BF16 && w->ne[0] == K && w->ne[2] == 1 && w->ne[3] == 1 && w->nb[0] == 2 && (w->nb[1] % 16) == 0 &&
+               !(((uintptr_t) w->data) & 15) && !buffer_is_split(w->buffer) && is_f32_contig(t) && !mm_cache_image_ok(t);
+    };
+    if (!eligible(n0)) return false;
+    std::vector<int> ms{i};
+    const int limit = std::min(g->n_nodes, i + 28);
+    for (int k = i + 1; k < limit && ms.size() < 4; ++k) {
+        const ggml_tensor * t = g->nodes[k];
+        if (st.done[k] || !eligible(t)) continue;
+        bool ok = true;
+        for (int mi : ms) ok = ok && !ranges_overlap(t, g->nodes[mi]);
+        for (int j = i + 1; j < k && ok; ++j) {  // everything that runs between node i and the sibling's own position
+            const ggml_tensor * u = g->nodes[j];
+            bool member = false;
+            for (int mi : ms) member = member || mi == j;
+            if (!is_view_op(u) && !member && ranges_overlap(t, u)) ok = false;
+            for (int sidx = 0; sidx < GGML_MAX_SRC && ok; ++sidx)
+                if (u->src[sidx] && ranges_overlap(t, u->src[sidx])) ok = false;
+        }
+        if (ok) ms.push_back(k);
+    }
+    if (ms.size() < 2) return false;
+    matvec_multi mm{};
+    mm.n = (int) ms.size();
+    double bytes = 0;
+    for (size_t q = 0; q < ms.size(); ++q) {
+        const ggml_tensor * t = g->nodes[ms[q]];
+        mm.W[q] = (const char *) t->src[0]->data;
+        mm.nb1[q] = (int64_t) t->src[0]->nb[1];
+        mm.N[q] = t->src[0]->ne[1];
+        mm.dst[q] = (float *) t->data;
+        bytes += (double) ggml_abi_nbytes(t->src[0]);
+    }
+    timed_scope ts(c, "mul_mat_f_siblings", bytes);
+    launch_matvec_bf16_multi(c->stream, mm, (const float *) X->data, K);
+    c->st.kernel_launches++;
+    for (size_t q = 1; q < ms.size(); ++q) { mark_done(st, ms[q]); c->st.fused_nodes++; }
+    return true;
+}
+
 // MUL(rows [n, n_used, T], w [1, n_used, T]) followed by the sum over the used experts written as views of the product and a chain of ADDs (one used
 // expert: a CONT of the one view): a single pass that writes the chain's last node.  Returns the number of nodes consumed (0: not that pattern).
 static int try_fuse_expert_sum(exec_state & st, int i) {
@@ -1828,6 +1880,7 @@ static int run_node(exec_state & st, int i) {
             }
             if (!is_quant(a->type) && fuse && c->opt.attn_nf && try_fuse_attn_nf(st, i)) return 1;
             if (!is_quant(a->type) && fuse && c->opt.attn_nf && try_fuse_attn_nf_mma(st, i)) return 1;
+            if (a->type == GGML_TYPE_BF16 && fuse && try_merge_matvec_bf16(st, i)) return 1;
             if (!is_quant(a->type)) {
                 timed_scope ts(c, "mul_mat_f", (double) ggml_abi_nbytes(a));
                 launch_mul_mat_f(s, TD(a), TD(b), TD(n), (float *) ((char *) c->ws + st.aux_off), c->ws ? c->ws_size - st.aux_off : 0);

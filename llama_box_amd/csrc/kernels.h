@@ -161,6 +161,9 @@ void launch_qkv(hipStream_t s, const qkv_args & a, int type_a, int type_b);
 // src1 rounded to f16 first when src0 is f16 (ggml-cpu vec_dot_type semantics)
 void launch_mul_mat_f(hipStream_t s, const tdesc & src0, const tdesc & src1, const tdesc & dst, float * ws = nullptr, size_t ws_bytes = 0);  // ws: scratch for K-split partial tiles
 size_t mul_mat_f_workspace_bytes(const tdesc & src0, const tdesc & src1);
+// up to four bf16 matrices (rows of K values, 16-byte aligned) against ONE f32 column of K values (K a multiple of 8), one launch
+struct matvec_multi { const char * W[4]; int64_t nb1[4]; int64_t N[4]; float * dst[4]; int blk0[5]; int n; };
+void launch_matvec_bf16_multi(hipStream_t s, matvec_multi mm, const float * x, int64_t K);
 // MUL_MAT_ID: as [K, N, n_expert] (f32 / f16 / bf16), b [K, 1 or n_used, T] f32, ids [n_used, T] i32 -> d [N, n_used, T].  ws: scratch for the
 // per-expert column lists of the batched form; lists_valid: an earlier call left the lists of these same ids there
 size_t mul_mat_id_workspace_bytes(const tdesc & as, const tdesc & ids);

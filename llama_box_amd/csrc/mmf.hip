@@ -931,6 +931,83 @@ __global__ void __launch_bounds__(256) k_mul_mat_id_mma(const tdesc a, const tde
     }
 }
 
+// a few columns (a decode step): four rows of the column's expert per workgroup, the four waves take slices of K with 16-byte loads (the form of
+// k_mul_mat_f16_gqa_long), so an expert's matrix streams at the rate of a plain mat-vec
+template <bool BF>
+__global__ void __launch_bounds__(256) k_mul_mat_id_vec(const tdesc a, const tdesc b, const tdesc ids, const tdesc d) {
+    __shared__ float part[4][4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t u = blockIdx.y, t = blockIdx.z, K = a.ne[0], row0 = (int64_t) blockIdx.x * 4;
+    const int32_t e = *(const int32_t *) (ids.data + u * ids.nb[0] + t * ids.nb[1]);
+    if (e < 0 || e >= a.ne[2]) return;
+    const char * wr[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) wr[r] = a.data + std::min<int64_t>(row0 + r, a.ne[1] - 1) * a.nb[1] + (int64_t) e * a.nb[2];
+    const char * xcol = b.data + (u % b.ne[1]) * b.nb[1] + t * b.nb[2];
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int64_t k = (int64_t) wave * 512 + lane * 8; k < K; k += 2048) {
+        float w[4][8], x[8];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) mmf_w8<BF>(wr[r] + k * 2, w[r]);
+        mmf_x8<BF>(xcol + k * 4, x);
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[r] = fmaf(w[r][i], x[i], acc[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const float v = wave_sum(acc[r]);
+        if (lane == 0) part[wave][r] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x < 4) {
+        const int r = threadIdx.x;
+        const float v = ((part[0][r] + part[1][r]) + part[2][r]) + part[3][r];
+        if (row0 + r < a.ne[1]) *(float *) (d.data + (row0 + r) * d.nb[0] + u * d.nb[1] + t * d.nb[2]) = v;
+    }
+}
+
+// up to four bf16 matrices against the same single column (a decode step's q / k / v / gate projections) in one launch: the workgroups are dealt over
+// the matrices' rows, four rows each, the waves taking slices of K (k_mul_mat_f16_gqa_long's form and arithmetic)
+__global__ void __launch_bounds__(256) k_matvec_bf16_multi(const matvec_multi mm, const char * __restrict__ x, const int64_t K) {
+    __shared__ float part[4][4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int q = 0;
+    while (q + 1 < mm.n && (int) blockIdx.x >= mm.blk0[q + 1]) ++q;
+    const int64_t row0 = (int64_t) ((int) blockIdx.x - mm.blk0[q]) * 4, N = mm.N[q];
+    const char * wr[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) wr[r] = mm.W[q] + std::min<int64_t>(row0 + r, N - 1) * mm.nb1[q];
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int64_t k = (int64_t) wave * 512 + lane * 8; k < K; k += 2048) {
+        float w[4][8], xv[8];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) mmf_w8<true>(wr[r] + k * 2, w[r]);
+        mmf_x8<true>(x + k * 4, xv);
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[r] = fmaf(w[r][i], xv[i], acc[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const float v = wave_sum(acc[r]);
+        if (lane == 0) part[wave][r] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x < 4) {
+        const int r = threadIdx.x;
+        const float v = ((part[0][r] + part[1][r]) + part[2][r]) + part[3][r];
+        if (row0 + r < N) mm.dst[q][row0 + r] = v;
+    }
+}
+void launch_matvec_bf16_multi(hipStream_t s, matvec_multi mm, const float * x, int64_t K) {
+    mm.blk0[0] = 0;
+    for (int q = 0; q < mm.n; ++q) mm.blk0[q + 1] = mm.blk0[q] + (int) ((mm.N[q] + 3) / 4);
+    hipLaunchKernelGGL(k_matvec_bf16_multi, dim3((unsigned) mm.blk0[mm.n]), dim3(256), 0, s, mm, (const char *) x, K);
+}
+
 size_t mul_mat_id_workspace_bytes(const tdesc & as, const tdesc & ids) {
     return ((size_t) as.ne[2] * 2 + (size_t) (ids.ne[0] * ids.ne[1])) * sizeof(int32_t) + 256;
 }
@@ -949,6 +1026,12 @@ void launch_mul_mat_id(hipStream_t s, const tdesc & as, const tdesc & b, const t
         const dim3 grid((unsigned) ((as.ne[1] + 63) / 64), (unsigned) std::max<int64_t>(1, std::min<int64_t>(64, (even + 63) / 64 * 2)), (unsigned) as.ne[2]);
         if (bf) hipLaunchKernelGGL(k_mul_mat_id_mma<true>, grid, dim3(256), 0, s, as, b, d, n_used, cnt, off, list);
         else hipLaunchKernelGGL(k_mul_mat_id_mma<false>, grid, dim3(256), 0, s, as, b, d, n_used, cnt, off, list);
+        return;
+    }
+    if (vec_ok && K >= 256) {
+        const dim3 grid((unsigned) ((as.ne[1] + 3) / 4), (unsigned) n_used, (unsigned) T);
+        if (bf) hipLaunchKernelGGL(k_mul_mat_id_vec<true>, grid, dim3(256), 0, s, as, b, ids, d);
+        else hipLaunchKernelGGL(k_mul_mat_id_vec<false>, grid, dim3(256), 0, s, as, b, ids, d);
         return;
     }
     int lpr = 64;

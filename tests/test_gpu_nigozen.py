@@ -213,6 +213,8 @@ def attention_case(backend, H, kv_type, n_q, n_kv, heads, kv_heads, dk, dv, chun
     mask[:n_q][ok] = 0.0
     if kv_type == L.BF16:
         k, v = R.bf16_round(k), R.bf16_round(v)
+        if n_q >= 32 and dk % 8 == 0 and dv % 8 == 0 and dk <= 128 and dv <= 128:
+            q = R.bf16_round(q)  # prompt portions over a bf16 cache run on the matrix cores: the queries are rounded to bf16 like every mat-mul operand
 
     def build(g):
         tq = g.new(L.F32, [dk, heads, n_q], q)
