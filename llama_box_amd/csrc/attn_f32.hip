@@ -222,7 +222,7 @@ __global__ void __launch_bounds__(256) k_attn_f32_tile(const tdesc q, const tdes
 }
 
 // ------------------------------------------------------------------------------------------------ prompt batches over a bf16 cache: the matrix cores
-// k_attn_mma_bf16: a workgroup owns 128 query tokens of one head, a wave 32 of them.  Per block of 32 cells
+// k_attn_mma_bf16: a wave owns 32 query tokens of one head; a workgroup is 1, 2 or 4 such waves sharing the staged V^T block.  Per block of 32 cells
 //   S^T = K . Q^T   on v_mfma_f32_32x32x16_bf16 (first operand: the cells' bf16 rows straight from the cache, 16 bytes a lane; second: the wave's queries,
 //                   rounded to bf16 once and kept in registers) — a lane then holds 16 scores of ITS query (its half-wave's cells), so the running maximum,
 //                   the sum and the rescaling are per-lane scalars and one exchange with the other half-wave;
@@ -230,7 +230,7 @@ __global__ void __launch_bounds__(256) k_attn_f32_tile(const tdesc q, const tdes
 //   O^T += V^T . P^T  on the same instruction, V^T staged through LDS (bf16, transposed on the way in), the weights P given as TWO bf16 terms
 //                   (p = hi + lo, |lo| <= 2^-9 |p|): the f32 weights enter the sum to 2^-17, not rounded to 8 bits.
 // The key order inside the second product is the order the first product's registers come in (both operands permuted alike).
-// Blocks that the mask hides from all 128 queries are skipped after the mask read.  Head sizes: multiples of 8 up to 16 DK16 / 32 DVT.
+// Blocks that the mask hides from all of a workgroup's queries are skipped after the mask read.  Head sizes: multiples of 8 up to 16 DK16 / 32 DVT.
 typedef __bf16 att_bf8 __attribute__((ext_vector_type(8)));
 typedef float att_f16v __attribute__((ext_vector_type(16)));
 __device__ __forceinline__ uint32_t att_bf16_bits(const float f) {
@@ -240,13 +240,13 @@ __device__ __forceinline__ uint32_t att_bf16_bits(const float f) {
 template <int DK16, int DVT>
 __global__ void __launch_bounds__(256) k_attn_mma_bf16(const tdesc q, const tdesc k, const tdesc v, const tdesc mask, const float * __restrict__ sinks, const tdesc dst, const float scale) {
     constexpr int VS = 36;  // V^T row stride in LDS (bf16 elements): 72 bytes keeps the 8-byte reads aligned and spreads the rows over the banks
-    __shared__ uint16_t Vt[DVT * 32 * VS];
+    __shared__ __attribute__((aligned(16))) uint16_t Vt[DVT * 32 * VS];
     __shared__ int flag[2];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 31, g = lane >> 5;
     const int64_t h = blockIdx.y, n_q = q.ne[1], n_kv = k.ne[1];
     const int DK = (int) q.ne[0], DV = (int) v.ne[0];
-    const int64_t tq = (int64_t) blockIdx.x * 128 + wave * 32 + n;  // this lane's query
+    const int64_t tq = (int64_t) blockIdx.x * (blockDim.x / 2) + wave * 32 + n;  // this lane's query (a workgroup of 1, 2 or 4 waves: 32 queries a wave)
     const bool q_live = tq < n_q;
     const int64_t kvh = h / (q.ne[2] / k.ne[2]);
     const char * kbase = k.data + kvh * k.nb[2];
@@ -273,10 +273,9 @@ __global__ void __launch_bounds__(256) k_attn_mma_bf16(const tdesc q, const tdes
     const char * mrow = mask.data + (q_live ? tq : 0) * mask.nb[1];
     if (threadIdx.x < 2) flag[threadIdx.x] = 0;
     __syncthreads();
-    for (int64_t j0 = 0, blk = 0; j0 < n_kv; j0 += 32, ++blk) {
-        // this lane's 16 mask terms: cells j0 + 8 b + 4 g .. + 3, b = 0 .. 3 (register i = 4 b + r)
-        float mv[16];
-        bool any = false;
+    // this lane's 16 mask terms of a block: cells j0 + 8 b + 4 g .. + 3, b = 0 .. 3 (register i = 4 b + r); the NEXT block's terms are requested while the
+    // current block is worked on (three dependent trips to memory per block — mask, V, K — were what bound this kernel)
+    auto load_mask = [&](const int64_t j0, float (&mv)[16]) {
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
             const int64_t j = j0 + 8 * b + 4 * g;
@@ -288,23 +287,49 @@ __global__ void __launch_bounds__(256) k_attn_mma_bf16(const tdesc q, const tdes
                 if (j + 2 < n_kv) t.z = ((const float *) mrow)[j + 2];
             }
             mv[4 * b] = t.x; mv[4 * b + 1] = t.y; mv[4 * b + 2] = t.z; mv[4 * b + 3] = t.w;
-            any = any || t.x > -INFINITY || t.y > -INFINITY || t.z > -INFINITY || t.w > -INFINITY;
         }
+    };
+    float mv_next[16];
+    load_mask(0, mv_next);
+    for (int64_t j0 = 0, blk = 0; j0 < n_kv; j0 += 32, ++blk) {
+        float mv[16];
+        bool any = false;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { mv[i] = mv_next[i]; any = any || mv[i] > -INFINITY; }
+        if (j0 + 32 < n_kv) load_mask(j0 + 32, mv_next);
         const bool wave_any = __ballot(any) != 0;
         if (threadIdx.x == 0) flag[(blk + 1) & 1] = 0;
         if (wave_any && lane == 0) flag[blk & 1] = 1;
         __syncthreads();
         if (!flag[blk & 1]) continue;  // (the same answer for every thread of the workgroup)
-        // V^T of the block into LDS: thread takes 8 consecutive value entries of one cell
-        for (int e0 = threadIdx.x; e0 < 32 * (DVT * 4); e0 += 256) {
-            const int cell = e0 / (DVT * 4), c8 = e0 % (DVT * 4);
-            uint4 t = make_uint4(0, 0, 0, 0);
-            if (j0 + cell < n_kv && 8 * c8 < DV) t = *(const uint4 *) (vbase + (j0 + cell) * v.nb[1] + c8 * 16);
-            const uint32_t u[4] = {t.x, t.y, t.z, t.w};
+        // the block's K operands are requested first, so that they travel while V^T is staged
+        uint4 kf[DK16];
+        {
+            const int64_t cell = j0 + n < n_kv ? j0 + n : n_kv - 1;
+            const char * krow = kbase + cell * k.nb[1] + g * 16;
+#pragma unroll
+            for (int s = 0; s < DK16; ++s) {
+                kf[s] = make_uint4(0, 0, 0, 0);
+                if (wave_any && 16 * s + 8 * g < DK) kf[s] = *(const uint4 *) (krow + s * 32);
+            }
+        }
+        // V^T of the block into LDS: a thread takes 8 consecutive value entries of FOUR neighbouring cells and writes eight 8-byte groups (4 cells of one entry)
+        for (int e0 = threadIdx.x; e0 < 8 * (DVT * 4); e0 += blockDim.x) {
+            const int cg = e0 / (DVT * 4), c8 = e0 % (DVT * 4);
+            uint32_t u[4][4];
+#pragma unroll
+            for (int cc = 0; cc < 4; ++cc) {
+                uint4 t = make_uint4(0, 0, 0, 0);
+                if (j0 + 4 * cg + cc < n_kv && 8 * c8 < DV) t = *(const uint4 *) (vbase + (j0 + 4 * cg + cc) * v.nb[1] + c8 * 16);
+                u[cc][0] = t.x; u[cc][1] = t.y; u[cc][2] = t.z; u[cc][3] = t.w;
+            }
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                Vt[(8 * c8 + 2 * e) * VS + cell] = (uint16_t) (u[e] & 0xFFFF);
-                Vt[(8 * c8 + 2 * e + 1) * VS + cell] = (uint16_t) (u[e] >> 16);
+                // entries 2 e (low halves) and 2 e + 1 (high halves) of the four cells
+                const uint2 lo2 = make_uint2((u[0][e] & 0xFFFFu) | (u[1][e] << 16), (u[2][e] & 0xFFFFu) | (u[3][e] << 16));
+                const uint2 hi2 = make_uint2((u[0][e] >> 16) | (u[1][e] & 0xFFFF0000u), (u[2][e] >> 16) | (u[3][e] & 0xFFFF0000u));
+                *(uint2 *) (Vt + (8 * c8 + 2 * e) * VS + 4 * cg) = lo2;
+                *(uint2 *) (Vt + (8 * c8 + 2 * e + 1) * VS + 4 * cg) = hi2;
             }
         }
         __syncthreads();
@@ -312,16 +337,8 @@ __global__ void __launch_bounds__(256) k_attn_mma_bf16(const tdesc q, const tdes
         att_f16v S;
 #pragma unroll
         for (int i = 0; i < 16; ++i) S[i] = 0.0f;
-        {
-            const int64_t cell = j0 + n < n_kv ? j0 + n : n_kv - 1;
-            const char * krow = kbase + cell * k.nb[1] + g * 16;
 #pragma unroll
-            for (int s = 0; s < DK16; ++s) {
-                uint4 kf = make_uint4(0, 0, 0, 0);
-                if (16 * s + 8 * g < DK) kf = *(const uint4 *) (krow + s * 32);
-                S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(att_bf8, kf), __builtin_bit_cast(att_bf8, qf[s]), S, 0, 0, 0);
-            }
-        }
+        for (int s = 0; s < DK16; ++s) S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(att_bf8, kf[s]), __builtin_bit_cast(att_bf8, qf[s]), S, 0, 0, 0);
         float mx = ATTN_F32_LOW;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
@@ -405,9 +422,16 @@ static void attn_f32_launch_t(hipStream_t s, const tdesc & q, const tdesc & k, c
     if constexpr (KT == GGML_TYPE_BF16 && VT == GGML_TYPE_BF16) {
         static const bool mma_on = !getenv("GGML_MI355X_ATTN_MMA") || atoi(getenv("GGML_MI355X_ATTN_MMA")) != 0;
         if (mma_on && attn_mma_bf16_ok(q, k, v, mask, dst)) {  // prompt portions over a bf16 cache: the matrix cores
-            const dim3 grid((unsigned) ((n_q + 127) / 128), (unsigned) H);
+            // waves per workgroup: four share a staged V^T block; two when four would leave most of the chip's 256 CUs without a workgroup (measured at 512 queries x 16
+            // heads: 1.87 ms for 16 launches with two waves, 2.12 with four, 1.99 with one)
+            int nw = ((n_q + 127) / 128) * H < 256 ? 2 : 4;
+            static const int nw_env = getenv("GGML_MI355X_ATTN_NW") ? atoi(getenv("GGML_MI355X_ATTN_NW")) : 0;
+            if (nw_env == 1 || nw_env == 2 || nw_env == 4) nw = nw_env;
+            while (nw > 1 && 32 * (nw / 2) >= n_q) nw >>= 1;  // (no more waves than the batch has groups of 32 queries)
+            const dim3 grid((unsigned) ((n_q + 32 * nw - 1) / (32 * nw)), (unsigned) H);
+            const dim3 block((unsigned) (64 * nw));
             const int dk16 = (DK + 15) / 16, dvt = (DV + 31) / 32;
-#define MI_ATT_MMA(A, B) hipLaunchKernelGGL((k_attn_mma_bf16<A, B>), grid, dim3(256), 0, s, q, k, v, *mask, sinks, dst, scale)
+#define MI_ATT_MMA(A, B) hipLaunchKernelGGL((k_attn_mma_bf16<A, B>), grid, block, 0, s, q, k, v, *mask, sinks, dst, scale)
             const int a = dk16 <= 2 ? 2 : (dk16 <= 4 ? 4 : 8), b = dvt <= 1 ? 1 : (dvt <= 2 ? 2 : 4);
             if (a == 2 && b == 1) MI_ATT_MMA(2, 1); else if (a == 2 && b == 2) MI_ATT_MMA(2, 2); else if (a == 2) MI_ATT_MMA(2, 4);
             else if (a == 4 && b == 1) MI_ATT_MMA(4, 1); else if (a == 4 && b == 2) MI_ATT_MMA(4, 2); else if (a == 4) MI_ATT_MMA(4, 4);

@@ -1792,6 +1792,30 @@ static int try_fuse_expert_sum(exec_state & st, int i) {
     return k - i;
 }
 
+// The SET_ROWS that stores tensor `src` (seen through views) into a cache kept in f32 / bf16, when it is src's ONLY reader and sits within the next nodes: its
+// node index, or -1.  Running it early, at src's own node, is legal: the cache rows are read by nothing before the store's own position, the indices are an input.
+static int sole_cache_store_of(const exec_state & st, int i, const ggml_tensor * src, int64_t n_tok) {
+    ggml_cgraph * g = st.g;
+    if (use_count(st, src) != 1 || (src->flags & GGML_TENSOR_FLAG_OUTPUT)) return -1;
+    const int limit = std::min(g->n_nodes, i + 16);
+    for (int k = i + 1; k < limit; ++k) {
+        const ggml_tensor * t = g->nodes[k];
+        if (st.done[k]) continue;
+        if (is_view_op(t)) {
+            if (through_views(t) == src && (use_count(st, t) != 1 || (t->flags & GGML_TENSOR_FLAG_OUTPUT))) return -1;
+            continue;
+        }
+        if (t->op != GGML_OP_SET_ROWS || through_views(t->src[0]) != src) continue;
+        const ggml_tensor * idx = t->src[1];
+        const bool type_ok = t->type == GGML_TYPE_F32 || t->type == GGML_TYPE_BF16;  // (an f16 cache has its own fused rope + store launch: try_fuse_rope_store)
+        if (!type_ok || t->nb[0] != ggml_abi_type_size(t->type) || t->ne[0] * n_tok != ggml_abi_nelements(src) || t->src[0]->ne[1] != n_tok || t->src[0]->ne[2] != 1 || t->src[0]->ne[3] != 1 ||
+            !ggml_abi_is_contiguous(t->src[0]) || idx->type != GGML_TYPE_I64 || !ggml_abi_is_contiguous(idx) || ggml_abi_nelements(idx) != n_tok || idx->op != GGML_OP_NONE)
+            return -1;
+        return k;
+    }
+    return -1;
+}
+
 static int run_node(exec_state & st, int i) {
     backend_ctx * c = st.c;
     ggml_cgraph * g = st.g;
@@ -2017,6 +2041,15 @@ static int run_node(exec_state & st, int i) {
             if (fuse && s2 && ad && s2->op == GGML_OP_SCALE && ad->op == GGML_OP_ADD && ((ad->src[0] == n && ad->src[1] == s2) || (ad->src[0] == s2 && ad->src[1] == n)) &&
                 ggml_abi_op_param_f32(n, 1) == 0.0f && ggml_abi_op_param_f32(s2, 1) == 0.0f && single_use(st, n) && single_use(st, s2) && is_f32_contig(s2->src[0]) && is_f32_contig(ad) &&
                 same_shape(n, s2) && same_shape(n, ad) && !(ranges_overlap(ad, a) && ad->data != a->data) && !(ranges_overlap(ad, s2->src[0]) && ad->data != s2->src[0]->data)) {
+                static const bool row_stores = !getenv("GGML_MI355X_ROW_STORES") || atoi(getenv("GGML_MI355X_ROW_STORES")) != 0;
+                const int ks = (row_stores && ad->ne[2] == 1 && ad->ne[3] == 1) ? sole_cache_store_of(st, i + 2, ad, ad->ne[1]) : -1;
+                if (ks >= 0) {  // the blend lives only in the cache
+                    const ggml_tensor * sr = g->nodes[ks];
+                    launch_axpby_store(s, (const float *) a->data, ggml_abi_op_param_f32(n, 0), (const float *) s2->src[0]->data, ggml_abi_op_param_f32(s2, 0), ad->ne[0], ad->ne[1],
+                                       (const int64_t *) sr->src[1]->data, TD(sr));
+                    mark_done(st, ks);
+                    c->st.fused_nodes++;
+                } else
                 launch_axpby(s, (const float *) a->data, ggml_abi_op_param_f32(n, 0), (const float *) s2->src[0]->data, ggml_abi_op_param_f32(s2, 0), (float *) ad->data, ggml_abi_nelements(ad));
                 c->st.kernel_launches++;
                 c->st.fused_nodes += 2;
@@ -2054,10 +2087,51 @@ static int run_node(exec_state & st, int i) {
             launch_unary(s, MI_UNARY_SQR, TD(a), TD(n));
             c->st.kernel_launches++;
             return 1;
-        case GGML_OP_ARGSORT:
+        case GGML_OP_ARGSORT: {
+            // a router: ARGSORT(desc) -> VIEW (top k) ... GET_ROWS(logits as [1, n, T], view) -> RESHAPE -> SOFT_MAX: one pass.  The last two sit a few nodes
+            // further on (the expert mat-muls that read the same view come first in the graph's order): they are executed early, here, which is legal when
+            // nothing in between reads or occupies the memory the weights are written to
+            if (fuse && n->op_params[0] == 1 && a->type == GGML_TYPE_F32 && a->ne[2] == 1 && a->ne[3] == 1 && ggml_abi_is_contiguous(n)) {
+                int kg = -1, ks = -1;
+                const int limit = std::min(g->n_nodes, i + 20);
+                for (int k = i + 1; k < limit && kg < 0; ++k) {
+                    const ggml_tensor * t = g->nodes[k];
+                    if (!st.done[k] && t->op == GGML_OP_GET_ROWS && t->src[1] && t->src[1]->view_src == n && t->src[1]->view_offs == 0) kg = k;
+                }
+                const ggml_tensor * gr = kg >= 0 ? g->nodes[kg] : nullptr;
+                if (gr && through_views(gr->src[0]) == a && gr->src[0]->ne[0] == 1 && gr->src[1]->ne[0] <= 256 && gr->src[1]->ne[1] == a->ne[1] && single_use(st, gr)) {
+                    for (int k = kg + 1; k < limit; ++k) {
+                        if (st.done[k]) break;
+                        if (is_view_op(g->nodes[k])) continue;
+                        if (g->nodes[k]->op == GGML_OP_SOFT_MAX) ks = k;
+                        break;
+                    }
+                }
+                const ggml_tensor * sm = ks >= 0 ? g->nodes[ks] : nullptr;
+                if (sm && through_views(sm->src[0]) == gr && !sm->src[1] && !sm->src[2] && ggml_abi_op_param_f32(sm, 0) == 1.0f && ggml_abi_op_param_f32(sm, 1) == 0.0f && is_f32_contig(sm) &&
+                    sm->ne[0] == gr->src[1]->ne[0] && sm->ne[1] == a->ne[1] && !ranges_overlap(sm, a) && !ranges_overlap(sm, n)) {
+                    bool ok = true;
+                    for (int j = i + 1; j < ks && ok; ++j) {
+                        const ggml_tensor * u = g->nodes[j];
+                        if (j == kg) continue;
+                        if (!is_view_op(u) && ranges_overlap(sm, u)) ok = false;
+                        for (int sidx = 0; sidx < GGML_MAX_SRC && ok; ++sidx)
+                            if (u->src[sidx] && u->src[sidx] != gr && ranges_overlap(sm, u->src[sidx])) ok = false;
+                    }
+                    if (ok) {
+                        launch_topk_softmax(s, TD(a), TD(n), TD(sm), (int) gr->src[1]->ne[0]);
+                        c->st.kernel_launches++;
+                        c->st.fused_nodes += 2;
+                        mark_done(st, kg);
+                        mark_done(st, ks);
+                        return 1;
+                    }
+                }
+            }
             launch_argsort(s, TD(a), TD(n), n->op_params[0] == 1 ? 1 : 0);
             c->st.kernel_launches++;
             return 1;
+        }
         case GGML_OP_NORM: {
             // NORM -> MUL(norm, w) [-> ADD(.., residual)]: one kernel writing the last node's output
             ggml_tensor * m = next(1);
@@ -2069,6 +2143,20 @@ static int run_node(exec_state & st, int i) {
                                                   ? (ad->src[0] == m ? ad->src[1] : (ad->src[1] == m ? ad->src[0] : nullptr)) : nullptr;
                     if (res && res->type == GGML_TYPE_F32 && res->nb[0] == 4 && same_shape(res, m) && !(ranges_overlap(ad, a) && ad->data != a->data)) {
                         const tdesc rd = TD(res);
+                        // ... [-> NORM(sum) -> MUL(.., w2)]: the norm in front of the next sublayer reads the row this kernel has just written
+                        ggml_tensor * n2 = next(3), * m2 = next(4);
+                        if (n2 && m2 && n2->op == GGML_OP_NORM && n2->src[0] == ad && m2->op == GGML_OP_MUL && single_use(st, n2) && m2->type == GGML_TYPE_F32 && m2->nb[0] == 4 &&
+                            same_shape(m2, ad) && !(ad->flags & GGML_TENSOR_FLAG_OUTPUT)) {
+                            const ggml_tensor * w2 = m2->src[0] == n2 ? m2->src[1] : (m2->src[1] == n2 ? m2->src[0] : nullptr);
+                            if (w2 && w2->type == GGML_TYPE_F32 && ggml_abi_is_contiguous(w2) && w2->ne[0] == n->ne[0] && ggml_abi_nelements(w2) == w2->ne[0] && !ranges_overlap(m2, ad) &&
+                                !(ranges_overlap(m2, a) && m2->data != a->data) && !ranges_overlap(m2, res)) {  // (a row's second output is written after the last read of that row of `a`: the allocator may hand `a`'s block to it)
+                                timed_scope ts(c, "layer_norm_mul_add_norm_mul", (double) ggml_abi_nbytes(a) * 4);
+                                launch_layer_norm_twice(s, TD(a), TD(ad), ggml_abi_op_param_f32(n, 0), (const float *) w->data, &rd, (const float *) w2->data, ggml_abi_op_param_f32(n2, 0), TD(m2));
+                                c->st.kernel_launches++;
+                                c->st.fused_nodes += 4;
+                                return 5;
+                            }
+                        }
                         timed_scope ts(c, "layer_norm_mul_add", (double) ggml_abi_nbytes(a) * 3);
                         launch_layer_norm(s, TD(a), TD(ad), ggml_abi_op_param_f32(n, 0), (const float *) w->data, &rd);
                         c->st.kernel_launches++;
@@ -2291,6 +2379,25 @@ static int run_node(exec_state & st, int i) {
         }
         case GGML_OP_ROPE: {
             if (fuse && try_fuse_rope_store(st, i)) return 1;
+            static const bool row_stores = !getenv("GGML_MI355X_ROW_STORES") || atoi(getenv("GGML_MI355X_ROW_STORES")) != 0;
+            if (fuse && row_stores && n->type == GGML_TYPE_F32 && a->type == GGML_TYPE_F32 && a->nb[0] == 4 && !(n->op_params[2] & GGML_ROPE_TYPE_MROPE) && !n->src[2] && n->ne[3] == 1 &&
+                ggml_abi_is_contiguous(n) && b->type == GGML_TYPE_I32) {
+                const int ks = sole_cache_store_of(st, i, n, n->ne[2]);
+                if (ks >= 0) {  // rope(k) lives only in the cache: rotate straight into the cache rows
+                    rope_params p;
+                    p.n_dims = n->op_params[1]; p.mode = n->op_params[2]; p.n_ctx_orig = n->op_params[4];
+                    p.freq_base = ggml_abi_op_param_f32(n, 5); p.freq_scale = ggml_abi_op_param_f32(n, 6); p.ext_factor = ggml_abi_op_param_f32(n, 7);
+                    p.attn_factor = ggml_abi_op_param_f32(n, 8); p.beta_fast = ggml_abi_op_param_f32(n, 9); p.beta_slow = ggml_abi_op_param_f32(n, 10);
+                    memset(p.sections, 0, sizeof(p.sections));
+                    const ggml_tensor * sr = g->nodes[ks];
+                    timed_scope ts(c, "rope_store_rows", (double) ggml_abi_nbytes(n) * 2);
+                    launch_rope_store(s, TD(a), TD(b), (const int64_t *) sr->src[1]->data, TD(sr), p);
+                    c->st.kernel_launches++;
+                    c->st.fused_nodes++;
+                    mark_done(st, ks);
+                    return 1;
+                }
+            }
             rope_params p;
             p.n_dims = n->op_params[1];
             p.mode = n->op_params[2];

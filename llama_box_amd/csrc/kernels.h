@@ -228,6 +228,8 @@ void launch_mmq(hipStream_t s, int type, const uint8_t * W, int64_t w_nb1, int K
 // ---- element-wise / normalisation / data movement (ops.hip)
 void launch_rms_norm(hipStream_t s, const tdesc & src, const tdesc & dst, float eps, const tdesc * mul_w /* optional fused weight */);
 void launch_layer_norm(hipStream_t s, const tdesc & src, const tdesc & dst, float eps, const float * mul_w /* optional fused weight */, const tdesc * residual /* optional fused ADD */);
+void launch_layer_norm_twice(hipStream_t s, const tdesc & src, const tdesc & dst, float eps, const float * mul_w, const tdesc * residual, const float * w2, float eps2, const tdesc & dst2);  // ... and dst2 = LN(dst) * w2
+void launch_topk_softmax(hipStream_t s, const tdesc & logits /* [n, T] */, const tdesc & ids /* [n, T] i32: the descending permutation */, const tdesc & wts /* [k, T] */, int k);  // k <= 256
 void launch_argsort(hipStream_t s, const tdesc & src, const tdesc & dst, int descending);  // rows of f32 -> i32 permutation (stable)
 // element-wise forms outside ggml's unary enumeration, served by launch_unary: x^2 (SQR) and relu(x)^2 (RELU followed by SQR)
 #define MI_UNARY_SQR 1000
@@ -305,6 +307,9 @@ void launch_rope_qk_store(hipStream_t s, rope_store_args a, int n_tokens);
 bool rope_qk_store_vec_ok(const rope_store_args & a, int n_tokens);
 void launch_rope_qk_store_vec(hipStream_t s, const rope_store_args & a, int n_tokens, const float * tab);
 void launch_rope(hipStream_t s, const tdesc & src, const tdesc & pos, const float * freq_factors, const tdesc & dst, const rope_params & p);
+// ROPE (no frequency factors) + SET_ROWS into a cache kept in f32 / f16 / bf16, and a x + b y + SET_ROWS: the value goes straight into cache row idx[t]
+void launch_rope_store(hipStream_t s, const tdesc & src /* [D, heads, T] f32 */, const tdesc & pos, const int64_t * idx, const tdesc & cache, const rope_params & p);
+void launch_axpby_store(hipStream_t s, const float * x, float a, const float * y, float b, int64_t n, int64_t n_tok, const int64_t * idx, const tdesc & cache);
 void launch_soft_max(hipStream_t s, const tdesc & src, const tdesc * mask, const float * sinks, const tdesc & dst, float scale, float max_bias);
 
 // ---- attention (fattn.hip)

@@ -136,7 +136,10 @@ void launch_rms_norm_mul_q80_panel(hipStream_t s, const tdesc & src, float eps, 
 // ------------------------------------------------------------------------------------------------ NORM (layer normalisation)
 // y = (x - mean) / sqrt(var + eps) [* w] [+ r], var = mean of the squared deviations (two passes over a row kept in registers / L2; sums in f64
 // like RMS_NORM's).  w: optional weight of the MUL that follows; r: optional residual rows of the ADD behind that (same shape as the output).
-__global__ void __launch_bounds__(256) k_layer_norm(const tdesc a, const tdesc d, const float eps, const float * __restrict__ w, const tdesc r, const int has_r) {
+// second stage (w2 != nullptr): the row just written is normalised once more into d2, y2 = LN(y) * w2 — the norm in front of the next sublayer, which reads
+// the residual stream this kernel has just updated (a thread re-reads the elements it wrote itself)
+__global__ void __launch_bounds__(256) k_layer_norm(const tdesc a, const tdesc d, const float eps, const float * __restrict__ w, const tdesc r, const int has_r,
+                                                    const float * __restrict__ w2 = nullptr, const float eps2 = 0.0f, const tdesc d2 = tdesc()) {
     __shared__ double sh[4];
     const int64_t row = blockIdx.x;
     const int64_t i1 = row % a.ne[1], i2 = (row / a.ne[1]) % a.ne[2], i3 = row / (a.ne[1] * a.ne[2]);
@@ -144,30 +147,139 @@ __global__ void __launch_bounds__(256) k_layer_norm(const tdesc a, const tdesc d
     float * __restrict__ y = (float *) (d.data + i1 * d.nb[1] + i2 * d.nb[2] + i3 * d.nb[3]);
     const float * __restrict__ rr = has_r ? (const float *) (r.data + i1 * r.nb[1] + i2 * r.nb[2] + i3 * r.nb[3]) : nullptr;
     const int64_t n = a.ne[0];
+    // rows of up to 4096 values are read ONCE and kept in registers (16 a thread); longer rows are re-read from L2 in every pass
+    constexpr int RC = 16;
+    const bool held = n <= 256 * RC;
+    float xv[RC];
     double s = 0.0;
-    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) s += (double) x[i];
+    if (held) {
+#pragma unroll
+        for (int u = 0; u < RC; ++u) {
+            const int64_t i = threadIdx.x + 256 * u;
+            xv[u] = i < n ? x[i] : 0.0f;
+            s += (double) xv[u];
+        }
+    } else {
+        for (int64_t i = threadIdx.x; i < n; i += blockDim.x) s += (double) x[i];
+    }
     s = block_sum_d(s, sh);
     const float mean = (float) (s / (double) n);
     __syncthreads();
     double q = 0.0;
-    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
-        const float dv = x[i] - mean;
-        q += (double) (dv * dv);
+    if (held) {
+#pragma unroll
+        for (int u = 0; u < RC; ++u) {
+            const float dv = xv[u] - mean;
+            if (threadIdx.x + 256 * u < n) q += (double) (dv * dv);
+        }
+    } else {
+        for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+            const float dv = x[i] - mean;
+            q += (double) (dv * dv);
+        }
     }
     q = block_sum_d(q, sh);
     const float var = (float) (q / (double) n);
     const float scale = 1.0f / sqrtf(var + eps);
-    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
-        float v = (x[i] - mean) * scale;
-        if (w) v *= w[i];
-        if (rr) v += rr[i];
-        y[i] = v;
+    double s2 = 0.0;
+    if (held) {
+#pragma unroll
+        for (int u = 0; u < RC; ++u) {
+            const int64_t i = threadIdx.x + 256 * u;
+            if (i < n) {
+                float v = (xv[u] - mean) * scale;
+                if (w) v *= w[i];
+                if (rr) v += rr[i];
+                y[i] = v;
+                xv[u] = v;
+                s2 += (double) v;
+            }
+        }
+    } else {
+        for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+            float v = (x[i] - mean) * scale;
+            if (w) v *= w[i];
+            if (rr) v += rr[i];
+            y[i] = v;
+            s2 += (double) v;
+        }
+    }
+    if (w2 == nullptr) return;
+    __syncthreads();
+    s2 = block_sum_d(s2, sh);
+    const float mean2 = (float) (s2 / (double) n);
+    __syncthreads();
+    double q2 = 0.0;
+    if (held) {
+#pragma unroll
+        for (int u = 0; u < RC; ++u) {
+            const float dv = xv[u] - mean2;
+            if (threadIdx.x + 256 * u < n) q2 += (double) (dv * dv);
+        }
+    } else {
+        for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+            const float dv = y[i] - mean2;
+            q2 += (double) (dv * dv);
+        }
+    }
+    q2 = block_sum_d(q2, sh);
+    const float scale2 = 1.0f / sqrtf((float) (q2 / (double) n) + eps2);
+    float * __restrict__ y2 = (float *) (d2.data + i1 * d2.nb[1] + i2 * d2.nb[2] + i3 * d2.nb[3]);
+    if (held) {
+#pragma unroll
+        for (int u = 0; u < RC; ++u) {
+            const int64_t i = threadIdx.x + 256 * u;
+            if (i < n) y2[i] = (xv[u] - mean2) * scale2 * w2[i];
+        }
+    } else {
+        for (int64_t i = threadIdx.x; i < n; i += blockDim.x) y2[i] = (y[i] - mean2) * scale2 * w2[i];
     }
 }
 void launch_layer_norm(hipStream_t s, const tdesc & src, const tdesc & dst, float eps, const float * mul_w, const tdesc * residual) {
     const int64_t rows = src.ne[1] * src.ne[2] * src.ne[3];
     if (rows == 0) return;
-    hipLaunchKernelGGL(k_layer_norm, dim3((unsigned) rows), dim3(256), 0, s, src, dst, eps, mul_w, residual ? *residual : src, residual ? 1 : 0);
+    hipLaunchKernelGGL(k_layer_norm, dim3((unsigned) rows), dim3(256), 0, s, src, dst, eps, mul_w, residual ? *residual : src, residual ? 1 : 0, (const float *) nullptr, 0.0f, src);
+}
+void launch_layer_norm_twice(hipStream_t s, const tdesc & src, const tdesc & dst, float eps, const float * mul_w, const tdesc * residual, const float * w2, float eps2, const tdesc & dst2) {
+    const int64_t rows = src.ne[1] * src.ne[2] * src.ne[3];
+    if (rows == 0) return;
+    hipLaunchKernelGGL(k_layer_norm, dim3((unsigned) rows), dim3(256), 0, s, src, dst, eps, mul_w, residual ? *residual : src, residual ? 1 : 0, w2, eps2, dst2);
+}
+
+// ------------------------------------------------------------------------------------------------ router: top-k and soft-max over the chosen logits
+// one workgroup per token: ranks by counting (k_argsort's stable order), the whole permutation is written (the top-k view reads its first columns), and the
+// soft-max over the k largest logits goes to `wts` [k, T] — ARGSORT, GET_ROWS of the chosen logits and SOFT_MAX in one pass
+__global__ void __launch_bounds__(256) k_topk_softmax(const tdesc a, const tdesc ids, const tdesc wts, const int k) {
+    __shared__ float top[256];
+    __shared__ float red[2];
+    const int64_t t = blockIdx.x;
+    const float * __restrict__ x = (const float *) (a.data + t * a.nb[1]);
+    int32_t * __restrict__ y = (int32_t *) (ids.data + t * ids.nb[1]);
+    const int n = (int) a.ne[0];
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const float v = x[i];
+        int before = 0;
+        for (int j = 0; j < n; ++j) {
+            const float u = x[j];
+            before += (u > v || (u == v && j < i)) ? 1 : 0;
+        }
+        y[before] = i;
+        if (before < k) top[before] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {  // k is a handful: the maximum is top[0], the sum runs in rank order
+        float sum = 0.0f;
+        for (int j = 0; j < k; ++j) sum += expf(top[j] - top[0]);
+        red[0] = top[0];
+        red[1] = sum;
+    }
+    __syncthreads();
+    float * __restrict__ wrow = (float *) (wts.data + t * wts.nb[1]);
+    for (int j = threadIdx.x; j < k; j += blockDim.x) wrow[j] = expf(top[j] - red[0]) / red[1];
+}
+void launch_topk_softmax(hipStream_t s, const tdesc & logits, const tdesc & ids, const tdesc & wts, int k) {
+    if (logits.ne[1] == 0) return;
+    hipLaunchKernelGGL(k_topk_softmax, dim3((unsigned) logits.ne[1]), dim3(256), 0, s, logits, ids, wts, k);
 }
 
 // ------------------------------------------------------------------------------------------------ ARGSORT
@@ -915,6 +1027,54 @@ void launch_rope(hipStream_t s, const tdesc & a, const tdesc & pos, const float 
     }
     if (a.type == GGML_TYPE_F16) hipLaunchKernelGGL(k_rope<true>, grid, dim3(64), 0, s, a, pos, ff, d, p, theta_scale, c0, c1);
     else hipLaunchKernelGGL(k_rope<false>, grid, dim3(64), 0, s, a, pos, ff, d, p, theta_scale, c0, c1);
+}
+
+// ROPE whose only reader is the SET_ROWS of a cache: the rotated head goes straight into its cache row (k_rope's arithmetic, then ONE rounding to the
+// cache's type — f32, f16 or bf16 — exactly what k_set_rows / the bf16 block kernel would store).  src [D, heads, T] f32; row idx[t] of the cache holds
+// heads x D values.
+__device__ __forceinline__ void store_as(char * __restrict__ row, const int type, const int64_t i, const float v) {
+    if (type == GGML_TYPE_F32) ((float *) row)[i] = v;
+    else if (type == GGML_TYPE_BF16) ((uint16_t *) row)[i] = f2bf(v);
+    else ((uint16_t *) row)[i] = f2h(v);
+}
+__global__ void __launch_bounds__(64) k_rope_store(const tdesc a, const tdesc pos, const int64_t * __restrict__ idx, char * __restrict__ cache, const int64_t cache_nb1, const int cache_type,
+                                                   const rope_params p, const float theta_scale, const float corr0, const float corr1) {
+    const int64_t i1 = blockIdx.x, i2 = blockIdx.y;
+    const int n_pairs = p.n_dims / 2;
+    const float pos_f = (float) *(const int32_t *) (pos.data + i2 * pos.nb[0]);
+    const float * __restrict__ src = (const float *) (a.data + i1 * a.nb[1] + i2 * a.nb[2]);
+    char * __restrict__ row = cache + idx[i2] * cache_nb1;
+    const int64_t base = i1 * a.ne[0];
+    const bool neox = (p.mode & GGML_ROPE_TYPE_NEOX) != 0;
+    for (int ip = threadIdx.x; ip < n_pairs; ip += blockDim.x) {
+        const int ia = neox ? ip : 2 * ip, ib = neox ? ip + n_pairs : 2 * ip + 1;
+        const float x0 = src[ia], x1 = src[ib];
+        float cs, sn;
+        rope_cos_sin(ip, pos_f, nullptr, rope_consts{theta_scale, p.freq_scale, p.ext_factor, p.attn_factor, corr0, corr1}, cs, sn);
+        store_as(row, cache_type, base + ia, x0 * cs - x1 * sn);
+        store_as(row, cache_type, base + ib, x0 * sn + x1 * cs);
+    }
+    for (int64_t i0 = p.n_dims + threadIdx.x; i0 < a.ne[0]; i0 += blockDim.x) store_as(row, cache_type, base + i0, src[i0]);
+}
+void launch_rope_store(hipStream_t s, const tdesc & a, const tdesc & pos, const int64_t * idx, const tdesc & cache, const rope_params & p) {
+    if (a.ne[1] * a.ne[2] == 0) return;
+    float theta_scale, c0, c1;
+    rope_host_consts(p, theta_scale, c0, c1);
+    hipLaunchKernelGGL(k_rope_store, dim3((unsigned) a.ne[1], (unsigned) a.ne[2]), dim3(64), 0, s, a, pos, idx, cache.data, cache.nb[1], cache.type, p, theta_scale, c0, c1);
+}
+// a x + b y (k_axpby's arithmetic) stored as rows of a cache: row t of n values goes to cache row idx[t]
+__global__ void __launch_bounds__(256) k_axpby_store(const float * __restrict__ x, const float a, const float * __restrict__ y, const float b, const int64_t n, const int64_t * __restrict__ idx,
+                                                     char * __restrict__ cache, const int64_t cache_nb1, const int cache_type) {
+    const int64_t t = blockIdx.x;
+    char * __restrict__ row = cache + idx[t] * cache_nb1;
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+        const float pp = x[t * n + i] * a, q = y[t * n + i] * b;
+        store_as(row, cache_type, i, pp + q);
+    }
+}
+void launch_axpby_store(hipStream_t s, const float * x, float a, const float * y, float b, int64_t n, int64_t n_tok, const int64_t * idx, const tdesc & cache) {
+    if (n_tok == 0) return;
+    hipLaunchKernelGGL(k_axpby_store, dim3((unsigned) n_tok), dim3(256), 0, s, x, a, y, b, n, idx, cache.data, cache.nb[1], cache.type);
 }
 
 // ------------------------------------------------------------------------------------------------ SOFT_MAX
