@@ -270,7 +270,7 @@ static ws_plan plan_ws(backend_ctx * c, const ggml_cgraph * g) {
         } else if (n->op == GGML_OP_MUL_MAT_ID && n->src[2]) {
             p.aux_bytes = std::max(p.aux_bytes, mul_mat_id_workspace_bytes(TD(n->src[0]), TD(n->src[2])));
         } else if (n->op == GGML_OP_FLASH_ATTN_EXT && fa_route(n) == 4) {
-            continue;  // the 32-bit kernel keeps its running sums on chip
+            continue;  // the 32-bit kernels keep their running sums on chip
         } else if (n->op == GGML_OP_FLASH_ATTN_EXT) {
             const tdesc q = TD(n->src[0]), k = TD(n->src[1]), v = TD(n->src[2]);
             // (both forms a 33+-token batch may take — matrix-core tiles or, for a mask known to be sparse, position lists — fit this)

@@ -853,32 +853,40 @@ __global__ void __launch_bounds__(256) k_mul_mat_id(const tdesc a, const tdesc b
     if (live && sl == 0) *(float *) (d.data + i01 * d.nb[0] + u * d.nb[1] + t * d.nb[2]) = acc;
 }
 
-// columns grouped by expert: cnt[e], off[e] (exclusive prefix) and list[off[e] + i] = u + n_used * t, in (t, u) order within an expert
+// columns grouped by expert: cnt[e], off[e] (exclusive prefix) and list[off[e] + i] = u + n_used * t, in (t, u) order within an expert.
+// One workgroup per expert: a first pass over the ids counts the columns of lower-numbered experts (-> off[e]) and its own (-> cnt[e]); a second pass
+// places its own columns in order (a ballot per wave, the waves' totals through LDS).  No atomics: the lists do not depend on timing.
 __global__ void __launch_bounds__(256) k_moe_group(const tdesc ids, const int n_expert, int32_t * __restrict__ cnt, int32_t * __restrict__ off, int32_t * __restrict__ list) {
-    __shared__ int32_t s_cnt[256], s_off[256];
+    __shared__ int s_less[4], s_eq[4], s_wave[4];
+    const int e = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t n_used = ids.ne[0], T = ids.ne[1], n = n_used * T;
-    // (thread e owns expert e: a scan of all columns per thread — a few thousand index reads from L2, no atomics, a deterministic order)
-    for (int e0 = 0; e0 < n_expert; e0 += 256) {
-        const int e = e0 + threadIdx.x;
-        int c = 0;
-        if (e < n_expert)
-            for (int64_t i = 0; i < n; ++i) c += *(const int32_t *) (ids.data + (i % n_used) * ids.nb[0] + (i / n_used) * ids.nb[1]) == e ? 1 : 0;
-        s_cnt[threadIdx.x] = c;
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            int base = e0 == 0 ? 0 : off[e0 - 1] + cnt[e0 - 1];
-            for (int x = 0; x < 256 && e0 + x < n_expert; ++x) { s_off[x] = base; base += s_cnt[x]; }
-        }
-        __syncthreads();
-        if (e < n_expert) {
-            cnt[e] = c;
-            off[e] = s_off[threadIdx.x];
-            int at = s_off[threadIdx.x];
-            for (int64_t i = 0; i < n; ++i)
-                if (*(const int32_t *) (ids.data + (i % n_used) * ids.nb[0] + (i / n_used) * ids.nb[1]) == e) list[at++] = (int32_t) i;
-        }
-        __syncthreads();
+    auto id_at = [&](const int64_t i) { return *(const int32_t *) (ids.data + (i % n_used) * ids.nb[0] + (i / n_used) * ids.nb[1]); };
+    int less = 0, eq = 0;
+    for (int64_t i = threadIdx.x; i < n; i += 256) {
+        const int32_t v = id_at(i);
+        less += (v >= 0 && v < e) ? 1 : 0;
+        eq += v == e ? 1 : 0;
     }
+    for (int o = 32; o > 0; o >>= 1) { less += __shfl_xor(less, o, 64); eq += __shfl_xor(eq, o, 64); }
+    if (lane == 0) { s_less[wave] = less; s_eq[wave] = eq; }
+    __syncthreads();
+    const int base = s_less[0] + s_less[1] + s_less[2] + s_less[3];
+    if (threadIdx.x == 0) { cnt[e] = s_eq[0] + s_eq[1] + s_eq[2] + s_eq[3]; off[e] = base; }
+    int placed = 0;
+    for (int64_t i0 = 0; i0 < n; i0 += 256) {
+        const int64_t i = i0 + threadIdx.x;
+        const bool mine = i < n && id_at(i) == e;
+        const uint64_t bal = __ballot(mine);
+        const int before = __popcll(bal & ((1ull << lane) - 1ull));
+        __syncthreads();
+        if (lane == 0) s_wave[wave] = __popcll(bal);
+        __syncthreads();
+        int wave_off = 0;
+        for (int w = 0; w < wave; ++w) wave_off += s_wave[w];
+        if (mine) list[base + placed + wave_off + before] = (int32_t) i;
+        placed += s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
+    }
+    (void) n_expert;
 }
 
 template <bool BF>
@@ -1020,7 +1028,7 @@ void launch_mul_mat_id(hipStream_t s, const tdesc & as, const tdesc & b, const t
     for (int i = 1; i < 3; ++i) vec_ok = vec_ok && (as.nb[i] % 16) == 0 && (b.nb[i] % 16) == 0;
     if (vec_ok && n_used * T >= 64 && as.ne[2] <= 65535 && ws && mul_mat_id_workspace_bytes(as, ids) <= ws_bytes) {
         int32_t * cnt = (int32_t *) ws, * off = cnt + as.ne[2], * list = off + as.ne[2];
-        if (!lists_valid) hipLaunchKernelGGL(k_moe_group, dim3(1), dim3(256), 0, s, ids, (int) as.ne[2], cnt, off, list);
+        if (!lists_valid) hipLaunchKernelGGL(k_moe_group, dim3((unsigned) as.ne[2]), dim3(256), 0, s, ids, (int) as.ne[2], cnt, off, list);
         // column tiles per expert in the grid: enough for an even spread (the loop inside covers an expert that drew more)
         const int64_t even = (n_used * T + as.ne[2] - 1) / as.ne[2];
         const dim3 grid((unsigned) ((as.ne[1] + 63) / 64), (unsigned) std::max<int64_t>(1, std::min<int64_t>(64, (even + 63) / 64 * 2)), (unsigned) as.ne[2]);

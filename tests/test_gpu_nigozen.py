@@ -375,3 +375,30 @@ def test_erf_gelu_and_squared_relu(backend, H):
     ge, rs = run(backend, build)
     assert np.abs(ge.reshape(-1) - R.gelu_erf(x.astype(np.float64))).max() <= 1e-6
     assert np.abs(rs.reshape(-1) - np.maximum(x.astype(np.float64), 0) ** 2).max() <= 1e-5
+
+
+def test_trace_run_command_line(tmp_path):
+    """bin/trace_run as a program: steps on standard input, one 'done <step>' line each, <step>.f32 only where logits were asked for"""
+    import os
+    import subprocess
+    import sys
+
+    cfg = cfg_b()
+    W = R.random_weights(cfg, 31)
+    model_dir, out_dir = str(tmp_path / "model"), str(tmp_path / "out")
+    R.write_model(model_dir, cfg, W)
+    t = toks(21, cfg["vocab"], 32)
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": t[:9], "want": [0, 8]}], "end": []},
+             {"step": 1, "entries": [{"id": "x", "tokens": t[9:20], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "x", "tokens": t[20:], "want": [0]}, {"id": "y", "tokens": t[:2], "want": [1]}], "end": ["x", "y"]}]
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bin", "trace_run")
+    p = subprocess.run([sys.executable, exe, "--model", model_dir, "--dtype", "float32", "--out", out_dir, "--max-tokens", "128"],
+                       input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [ln for ln in p.stdout.splitlines() if ln.startswith("done")] == ["done 0", "done 1", "done 2"]
+    assert sorted(os.listdir(out_dir)) == ["0.f32", "2.f32"]
+    ref = R.forward(cfg, W, t)
+    r0 = np.fromfile(os.path.join(out_dir, "0.f32"), dtype="<f4").reshape(2, -1)
+    r2 = np.fromfile(os.path.join(out_dir, "2.f32"), dtype="<f4").reshape(2, -1)
+    assert row_err(r0, ref[[0, 8]]).max() <= F32_GATE
+    assert row_err(r2, np.stack([ref[20], ref[1]])).max() <= F32_GATE  # request y repeats x's first tokens in its own slot
