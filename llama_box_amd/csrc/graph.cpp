@@ -2184,9 +2184,9 @@ static int run_node(exec_state & st, int i) {
             const size_t need = mul_mat_id_workspace_bytes(TD(a), TD(ids));
             void * ws = (c->ws && st.aux_off + need <= c->ws_size) ? (char *) c->ws + st.aux_off : nullptr;
             timed_scope ts(c, "mul_mat_id", (double) ggml_abi_nbytes(a) / (double) std::max<int64_t>(1, a->ne[2]) * (double) std::min<int64_t>(a->ne[2], ggml_abi_nelements(ids)));
-            launch_mul_mat_id(s, TD(a), TD(b), TD(ids), TD(n), ws, ws ? c->ws_size - st.aux_off : 0, valid && ws);
-            st.moe_ids = ws ? ids : nullptr;
-            st.moe_node = i;
+            const bool grouped = launch_mul_mat_id(s, TD(a), TD(b), TD(ids), TD(n), ws, ws ? c->ws_size - st.aux_off : 0, valid && ws);
+            st.moe_ids = grouped ? ids : nullptr;  // (only a launch that made or used the lists vouches for them: the per-column forms leave the scratch alone)
+            st.moe_node = grouped ? i : -1;
             c->st.kernel_launches++;
             return 1;
         }

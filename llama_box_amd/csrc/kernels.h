@@ -167,7 +167,7 @@ void launch_matvec_bf16_multi(hipStream_t s, matvec_multi mm, const float * x, i
 // MUL_MAT_ID: as [K, N, n_expert] (f32 / f16 / bf16), b [K, 1 or n_used, T] f32, ids [n_used, T] i32 -> d [N, n_used, T].  ws: scratch for the
 // per-expert column lists of the batched form; lists_valid: an earlier call left the lists of these same ids there
 size_t mul_mat_id_workspace_bytes(const tdesc & as, const tdesc & ids);
-void launch_mul_mat_id(hipStream_t s, const tdesc & as, const tdesc & b, const tdesc & ids, const tdesc & d, void * ws, size_t ws_bytes, bool lists_valid);
+bool launch_mul_mat_id(hipStream_t s, const tdesc & as, const tdesc & b, const tdesc & ids, const tdesc & d, void * ws, size_t ws_bytes, bool lists_valid);  // true: the batched form ran and left the lists in ws
 // FLASH_ATTN_EXT in 32-bit arithmetic over f32 / bf16 / f16 K and V read in place, any head sizes up to 256, K and V sizes independent (attn_f32.hip)
 bool attn_f32_applies(const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const tdesc & dst);
 void launch_attn_f32(hipStream_t s, const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const float * sinks, const tdesc & dst, float scale);

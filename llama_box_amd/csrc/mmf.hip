@@ -1020,9 +1020,10 @@ size_t mul_mat_id_workspace_bytes(const tdesc & as, const tdesc & ids) {
     return ((size_t) as.ne[2] * 2 + (size_t) (ids.ne[0] * ids.ne[1])) * sizeof(int32_t) + 256;
 }
 // grouped: the column lists made by an earlier call over the same ids (the down projection follows the up projection) are used again
-void launch_mul_mat_id(hipStream_t s, const tdesc & as, const tdesc & b, const tdesc & ids, const tdesc & d, void * ws, size_t ws_bytes, bool lists_valid) {
+// returns true when the batched form ran: the column lists of these ids are then in ws (false: ws was not touched)
+bool launch_mul_mat_id(hipStream_t s, const tdesc & as, const tdesc & b, const tdesc & ids, const tdesc & d, void * ws, size_t ws_bytes, bool lists_valid) {
     const int64_t K = as.ne[0], n_used = ids.ne[0], T = ids.ne[1];
-    if (as.ne[1] == 0 || n_used * T == 0) return;
+    if (as.ne[1] == 0 || n_used * T == 0) return false;
     const bool bf = as.type == GGML_TYPE_BF16, w16 = bf || as.type == GGML_TYPE_F16;
     bool vec_ok = w16 && as.nb[0] == 2 && b.nb[0] == 4 && (K % 8) == 0 && (((uintptr_t) as.data) & 15) == 0 && (((uintptr_t) b.data) & 15) == 0;
     for (int i = 1; i < 3; ++i) vec_ok = vec_ok && (as.nb[i] % 16) == 0 && (b.nb[i] % 16) == 0;
@@ -1034,13 +1035,13 @@ void launch_mul_mat_id(hipStream_t s, const tdesc & as, const tdesc & b, const t
         const dim3 grid((unsigned) ((as.ne[1] + 63) / 64), (unsigned) std::max<int64_t>(1, std::min<int64_t>(64, (even + 63) / 64 * 2)), (unsigned) as.ne[2]);
         if (bf) hipLaunchKernelGGL(k_mul_mat_id_mma<true>, grid, dim3(256), 0, s, as, b, d, n_used, cnt, off, list);
         else hipLaunchKernelGGL(k_mul_mat_id_mma<false>, grid, dim3(256), 0, s, as, b, d, n_used, cnt, off, list);
-        return;
+        return true;
     }
     if (vec_ok && K >= 256) {
         const dim3 grid((unsigned) ((as.ne[1] + 3) / 4), (unsigned) n_used, (unsigned) T);
         if (bf) hipLaunchKernelGGL(k_mul_mat_id_vec<true>, grid, dim3(256), 0, s, as, b, ids, d);
         else hipLaunchKernelGGL(k_mul_mat_id_vec<false>, grid, dim3(256), 0, s, as, b, ids, d);
-        return;
+        return false;
     }
     int lpr = 64;
     while (lpr > 8 && (int64_t) (lpr / 2) >= K) lpr >>= 1;
@@ -1049,6 +1050,7 @@ void launch_mul_mat_id(hipStream_t s, const tdesc & as, const tdesc & b, const t
     if (bf) hipLaunchKernelGGL(k_mul_mat_id<2>, grid, dim3(256), 0, s, as, b, ids, d, lpr);
     else if (w16) hipLaunchKernelGGL(k_mul_mat_id<1>, grid, dim3(256), 0, s, as, b, ids, d, lpr);
     else hipLaunchKernelGGL(k_mul_mat_id<0>, grid, dim3(256), 0, s, as, b, ids, d, lpr);
+    return false;
 }
 
 MI_TU_TOUCH(mmf)

@@ -1144,8 +1144,13 @@ static void make_inputs(llm_context * c, ggml_context * ctx, int l0, int l1, boo
         io.resid = ggml_new_tensor_2d(ctx, GGML_TYPE_F32, hp.n_embd, n_tokens);
         ggml_set_input(named(io.resid, "l_out_from_the_previous_device", -1));
     }
-    io.pos = ggml_new_tensor_1d(ctx, GGML_TYPE_I32, n_tokens);
-    ggml_set_input(named(io.pos, "inp_pos", -1));
+    // (a model none of whose layers rotates has no reader of the positions: the input is then not made — the graph allocator places only what the graph reaches)
+    bool need_pos = m->lcfg.empty();
+    for (const llm_layer_cfg & lc : m->lcfg) need_pos = need_pos || lc.rot_dims > 0;
+    if (need_pos) {
+        io.pos = ggml_new_tensor_1d(ctx, GGML_TYPE_I32, n_tokens);
+        ggml_set_input(named(io.pos, "inp_pos", -1));
+    }
     const int64_t n_tok_pad = (n_tokens + 63) / 64 * 64;  // GGML_KQ_MASK_PAD
     // llama.cpp's build_attn_inp_kv_unified: the mask is an F32 input filled on the host; with flash attention FLASH_ATTN_EXT is handed a
     // ggml_cast(F16) of it (self_kq_mask_cnv) — a CPY node in the graph, not an F16 upload
@@ -1813,7 +1818,7 @@ static int decode_ubatch(llm_context * c, int n_tokens, const int32_t * tokens, 
         else ggml_backend_tensor_set(t, dst, 0, bytes);
     };
     upload(c->inp_tokens, (size_t) n_tokens * 4, [&](char * d) { memcpy(d, tokens, (size_t) n_tokens * 4); });
-    upload(c->inp_pos, (size_t) n_tokens * 4, [&](char * d) { memcpy(d, pos, (size_t) n_tokens * 4); });
+    if (c->inp_pos) upload(c->inp_pos, (size_t) n_tokens * 4, [&](char * d) { memcpy(d, pos, (size_t) n_tokens * 4); });
     upload(c->inp_k_idxs, (size_t) n_tokens * 8, [&](char * d) {
         int64_t * k = (int64_t *) d;
         for (int i = 0; i < n_tokens; ++i) k[i] = slots[i];

@@ -59,7 +59,13 @@ def cfg_b(dtype="f32"):
     ], eps=1e-6, embed_scale=0.25)
 
 
-CONFIGS = {"a": cfg_a, "b": cfg_b}
+def cfg_c(dtype="f32"):
+    # a single layer that does not rotate (no reader of the positions in the whole graph), rows of 36 values, an odd vocabulary
+    return R.make_config(36, 257, [dict(heads=2, kv_heads=2, dim=8, vdim=32, rot_dims=0, scale=0.25, chunk=33, v_mix=True, mlp=("moe", 16, 5, 2) if dtype == "f32" else ("moe", 16, 2, 2))],
+                         eps=1e-5, embed_scale=0.5)
+
+
+CONFIGS = {"a": cfg_a, "b": cfg_b, "c": cfg_c}
 
 
 class Served:
@@ -83,7 +89,7 @@ def toks(n, vocab, seed):
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
-@pytest.mark.parametrize("which", ["a", "b"])
+@pytest.mark.parametrize("which", ["a", "b", "c"])
 def test_whole_prompt(backend, tmp_path, plog, which, dtype):
     s = Served(backend, tmp_path, CONFIGS[which](dtype), 11, dtype)
     t = toks(150, s.cfg["vocab"], 5)  # three micro-batches of 64 / 64 / 22 tokens; every position's logits
@@ -108,7 +114,7 @@ def test_prefill_against_token_by_token(backend, tmp_path, dtype):
     s.free()
 
 
-@pytest.mark.parametrize("which", ["a", "b"])
+@pytest.mark.parametrize("which", ["a", "b", "c"])
 def test_portions_of_every_size(backend, tmp_path, which):
     s = Served(backend, tmp_path, CONFIGS[which](), 13, "f32")
     t = toks(131, s.cfg["vocab"], 7)
@@ -332,7 +338,9 @@ def test_mat_mul_with_bf16_and_f32_matrices(backend, H, wtype, K, N, M):
 
 
 @pytest.mark.parametrize("wtype", [L.F32, L.BF16])
-@pytest.mark.parametrize("T_,E,ff,n_exp,top", [(1, 64, 24, 5, 2), (3, 52, 12, 2, 2), (90, 64, 40, 6, 3), (200, 128, 64, 8, 1)])
+@pytest.mark.parametrize("T_,E,ff,n_exp,top", [(1, 64, 24, 5, 2), (3, 52, 12, 2, 2), (90, 64, 40, 6, 3), (200, 128, 64, 8, 1),
+                                               (90, 36, 24, 5, 2),     # rows of 36 values: the up projection runs column by column, the down projection (24) grouped by expert
+                                               (70, 64, 12, 3, 3)])    # ... and the other way round
 def test_experts_router_and_weighted_sum(backend, H, wtype, T_, E, ff, n_exp, top):
     """the whole mixture-of-experts block as the engine builds it: router logits, the top entries, soft-max over them, squared-ReLU experts, the weighted sum"""
     rng = np.random.default_rng(T_ + E)

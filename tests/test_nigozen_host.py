@@ -131,3 +131,13 @@ def test_reference_attention_edges():
     assert np.allclose(p, [[1 / 3, 1 / 3, 0.0]])
     x = R.rotate_pairs(np.ones((1, 1, 6)), [3], 4, 100.0)
     assert np.allclose(x[0, 0, 4:], 1.0) and np.allclose(x[0, 0, 0], np.cos(3) - np.sin(3)) and np.allclose(x[0, 0, 3], np.cos(0.3) + np.sin(0.3))
+
+
+def test_a_model_without_rotary_layers_has_no_position_input(H):
+    """no layer rotates -> nothing reads the positions: the engine must not upload into an input the graph allocator never placed"""
+    cfg = R.make_config(36, 57, [dict(heads=2, kv_heads=2, dim=8, vdim=32, rot_dims=0, scale=0.25, chunk=33, v_mix=True, mlp=("moe", 16, 5, 2))])
+    m = H.llm_model_synth_config(json.dumps(cfg).encode(), 1, H.ggml_backend_cpu_buffer_type(), L.BF16)
+    assert m
+    seen = _graph_probe(H, m, 256, [([1, 2, 3, 4, 5], [0, 1, 2, 3, 4], [0] * 5), ([6], [5], [0])])
+    assert len(seen) == 2 and "ROPE" not in seen[0][0]
+    H.llm_model_free(m)
