@@ -168,6 +168,14 @@ __device__ __forceinline__ void rope_yarn_dev(const float theta, const int ip, c
     cs = cosf(th) * mscale;
     sn = sinf(th) * mscale;
 }
+// the angle of pair ip as pos * base^(-2 ip / n_dims) with the frequency itself correct to an f32 rounding (computed in f64): one rounding of the frequency and one of
+// the product, instead of the ip accumulated roundings of the recurrence below.  For graphs that ask for it (ROPE op_params[3] == 1; no scaling, no YaRN, no factors).
+__device__ __forceinline__ void rope_cos_sin_exact(const int ip, const float pos_f, const float freq_base, const int n_dims, float & cs, float & sn) {
+    const float f = (float) pow((double) freq_base, -2.0 * (double) ip / (double) n_dims);
+    const float theta = pos_f * f;
+    cs = cosf(theta);
+    sn = sinf(theta);
+}
 __device__ __forceinline__ void rope_cos_sin(const int ip, const float pos_f, const float * __restrict__ ff, const rope_consts rc, float & cs, float & sn) {
     float theta = pos_f;
     for (int k = 0; k < ip; ++k) theta *= rc.theta_scale;

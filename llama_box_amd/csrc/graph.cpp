@@ -115,6 +115,13 @@ static int fa_route(const ggml_tensor * op) {
 // f32 rows that kv_types.hip can turn into bf16 a block of 32 values at a time (whole blocks, 16-byte aligned rows); others go element by element
 static bool bf16_rows_in_blocks(const ggml_tensor * a) { return (a->ne[0] % 32) == 0 && (a->nb[1] % 16) == 0 && (a->nb[2] % 16) == 0 && (a->nb[3] % 16) == 0; }
 
+// ROPE op_params[3] (ggml's unused n_ctx slot) == 1: the graph asks for per-pair frequencies computed on their own (dev_util.h: rope_cos_sin_exact); honoured for the
+// plain case only (no frequency scaling, no YaRN, no factors, not multi-section)
+static int rope_exact_freq(const ggml_tensor * n) {
+    return (n->op_params[3] == 1 && !n->src[2] && !(n->op_params[2] & GGML_ROPE_TYPE_MROPE) && ggml_abi_op_param_f32(n, 6) == 1.0f && ggml_abi_op_param_f32(n, 7) == 0.0f &&
+            ggml_abi_op_param_f32(n, 8) == 1.0f) ? 1 : 0;
+}
+
 bool supports_op(const ggml_tensor * op) {
     const ggml_tensor * a = op->src[0];
     const ggml_tensor * b = op->src[1];
@@ -1384,6 +1391,7 @@ static bool plan_rope_store(const exec_state & st, int i, rope_store_plan & pl) 
     ggml_cgraph * g = st.g;
     const ggml_tensor * rq = g->nodes[i];
     if (rq->op != GGML_OP_ROPE) return false;
+    if (rq->op_params[3] == 1) return false;  // (exact per-pair frequencies: served by the plain rope kernels)
     const ggml_tensor * q = rq->src[0];
     if (rq->type != GGML_TYPE_F32 || !ggml_abi_is_contiguous(rq) || q->type != GGML_TYPE_F32 || q->nb[0] != 4 || rq->ne[3] != 1 || rq->ne[2] < 2) return false;
     if ((rq->op_params[2] & GGML_ROPE_TYPE_MROPE) || rq->src[1]->type != GGML_TYPE_I32 || !ggml_abi_is_contiguous(rq->src[1])) return false;
@@ -2389,6 +2397,7 @@ static int run_node(exec_state & st, int i) {
                     p.freq_base = ggml_abi_op_param_f32(n, 5); p.freq_scale = ggml_abi_op_param_f32(n, 6); p.ext_factor = ggml_abi_op_param_f32(n, 7);
                     p.attn_factor = ggml_abi_op_param_f32(n, 8); p.beta_fast = ggml_abi_op_param_f32(n, 9); p.beta_slow = ggml_abi_op_param_f32(n, 10);
                     memset(p.sections, 0, sizeof(p.sections));
+                    p.exact_freq = rope_exact_freq(n);
                     const ggml_tensor * sr = g->nodes[ks];
                     timed_scope ts(c, "rope_store_rows", (double) ggml_abi_nbytes(n) * 2);
                     launch_rope_store(s, TD(a), TD(b), (const int64_t *) sr->src[1]->data, TD(sr), p);
@@ -2409,6 +2418,7 @@ static int run_node(exec_state & st, int i) {
             p.beta_fast = ggml_abi_op_param_f32(n, 9);
             p.beta_slow = ggml_abi_op_param_f32(n, 10);
             memcpy(p.sections, n->op_params + 11, sizeof(p.sections));
+            p.exact_freq = rope_exact_freq(n);
             timed_scope ts(c, "rope", (double) ggml_abi_nbytes(n) * 2);
             launch_rope(s, TD(a), TD(b), n->src[2] ? (const float *) n->src[2]->data : nullptr, TD(n), p);
             c->st.kernel_launches++;

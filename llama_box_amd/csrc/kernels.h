@@ -277,6 +277,7 @@ struct rope_params {
     int n_dims, mode, n_ctx_orig;
     float freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow;
     int sections[4];  // ggml_rope_multi (mode & GGML_ROPE_TYPE_MROPE): pairs per position stream (time, height, width, extra)
+    int exact_freq = 0;  // 1: every pair's frequency base^(-2 i / n_dims) is computed on its own (f64, rounded once) instead of by the recurrence theta *= theta_scale
 };
 void rope_host_consts(const rope_params & p, float & theta_scale, float & corr0, float & corr1);
 // (cos, sin) of every (token, rotation pair) of a small batch — rope_cos_sin's arithmetic, once per graph run instead of once per layer and element

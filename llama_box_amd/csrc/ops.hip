@@ -681,7 +681,8 @@ template <bool F16IO> __global__ void __launch_bounds__(64) k_rope(const tdesc a
         if (F16IO) { x0 = h2f(((const uint16_t *) src)[ia]); x1 = h2f(((const uint16_t *) src)[ib]); }
         else { x0 = ((const float *) src)[ia]; x1 = ((const float *) src)[ib]; }
         float cs, sn;
-        rope_cos_sin(ip, pos_f, ff, rope_consts{theta_scale, p.freq_scale, p.ext_factor, p.attn_factor, corr0, corr1}, cs, sn);
+        if (p.exact_freq) rope_cos_sin_exact(ip, pos_f, p.freq_base, p.n_dims, cs, sn);
+        else rope_cos_sin(ip, pos_f, ff, rope_consts{theta_scale, p.freq_scale, p.ext_factor, p.attn_factor, corr0, corr1}, cs, sn);
         if (F16IO) {
             ((uint16_t *) dst)[ia] = f2h(x0 * cs - x1 * sn);
             ((uint16_t *) dst)[ib] = f2h(x0 * sn + x1 * cs);
@@ -1050,7 +1051,8 @@ __global__ void __launch_bounds__(64) k_rope_store(const tdesc a, const tdesc po
         const int ia = neox ? ip : 2 * ip, ib = neox ? ip + n_pairs : 2 * ip + 1;
         const float x0 = src[ia], x1 = src[ib];
         float cs, sn;
-        rope_cos_sin(ip, pos_f, nullptr, rope_consts{theta_scale, p.freq_scale, p.ext_factor, p.attn_factor, corr0, corr1}, cs, sn);
+        if (p.exact_freq) rope_cos_sin_exact(ip, pos_f, p.freq_base, p.n_dims, cs, sn);
+        else rope_cos_sin(ip, pos_f, nullptr, rope_consts{theta_scale, p.freq_scale, p.ext_factor, p.attn_factor, corr0, corr1}, cs, sn);
         store_as(row, cache_type, base + ia, x0 * cs - x1 * sn);
         store_as(row, cache_type, base + ib, x0 * sn + x1 * cs);
     }

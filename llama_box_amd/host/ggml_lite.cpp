@@ -545,6 +545,12 @@ struct ggml_tensor * ggml_flash_attn_ext(struct ggml_context * ctx, struct ggml_
     r->src[3] = mask;
     return r;
 }
+// harness extension: asks the backend to compute every rotation pair's frequency base^(-2 i / n_dims) on its own instead of by ggml's recurrence
+// (theta *= theta_scale accumulates one rounding per pair): op_params[3], ggml's unused n_ctx slot
+void ggml_rope_set_exact_freq(struct ggml_tensor * a) {
+    LITE_ASSERT(a->op == GGML_OP_ROPE);
+    a->op_params[3] = 1;
+}
 void ggml_flash_attn_ext_set_prec(struct ggml_tensor * a, enum ggml_prec prec) {
     LITE_ASSERT(a->op == GGML_OP_FLASH_ATTN_EXT);
     a->op_params[3] = (int32_t) prec;

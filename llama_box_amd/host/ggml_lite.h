@@ -103,6 +103,7 @@ struct ggml_tensor * ggml_rope_multi(struct ggml_context * ctx, struct ggml_tens
 struct ggml_tensor * ggml_rope_ext_inplace(struct ggml_context * ctx, struct ggml_tensor * a, struct ggml_tensor * b, struct ggml_tensor * c,
                                    int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale, float ext_factor,
                                    float attn_factor, float beta_fast, float beta_slow);
+void ggml_rope_set_exact_freq(struct ggml_tensor * a);
 struct ggml_tensor * ggml_flash_attn_ext(struct ggml_context * ctx, struct ggml_tensor * q, struct ggml_tensor * k, struct ggml_tensor * v,
                                          struct ggml_tensor * mask, float scale, float max_bias, float logit_softcap);
 void ggml_flash_attn_ext_set_prec(struct ggml_tensor * a, enum ggml_prec prec);

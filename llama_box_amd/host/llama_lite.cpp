@@ -1314,6 +1314,8 @@ static void build_layerwise(llm_context * c, ggml_context * ctx, ggml_cgraph * g
         if (lc.rot_dims > 0) {  // neighbouring pairs (2i, 2i + 1) of the leading rot_dims entries; the rest of the head passes through
             Qcur = named(ggml_rope_ext(ctx, Qcur, io.pos, nullptr, lc.rot_dims, 0, hp.n_ctx_train, lc.rot_base, 1.0f, 0.0f, 1.0f, 32.0f, 1.0f), "Qcur_rope", il);
             Kcur = named(ggml_rope_ext(ctx, Kcur, io.pos, nullptr, lc.rot_dims, 0, hp.n_ctx_train, lc.rot_base, 1.0f, 0.0f, 1.0f, 32.0f, 1.0f), "Kcur_rope", il);
+            ggml_rope_set_exact_freq(Qcur);  // angle = pos * base^(-2 i / dims) with the frequency itself rounded once (not ggml's running product)
+            ggml_rope_set_exact_freq(Kcur);
         }
         if (lc.v_mix) {
             if (!v_first) v_first = Vcur;
