@@ -42,6 +42,34 @@ __device__ __forceinline__ float mask_ld(const char * __restrict__ mrow, const i
     return mtype == GGML_TYPE_F16 ? h2f(((const uint16_t *) mrow)[j]) : ((const float *) mrow)[j];
 }
 
+// acc[r] += sum over the block's visible cells of p[cell] * V[cell][lane + 64 r]: no branches around the loads (a lane beyond the row's end re-reads the last
+// column, its sum is dropped later; hidden cells enter with weight 0)
+template <int VT, int CELLS, int RR>
+__device__ __forceinline__ void attn_f32_pv(const float p, const uint64_t live, const char * __restrict__ vbase, const int64_t v_nb1, const int64_t j0, const int64_t n_kv, const int DV,
+                                            const int lane, float (&acc)[ATTN_F32_MAX_D / 64]) {
+    const uint64_t gmask = CELLS == 64 ? ~0ull : ((1ull << CELLS) - 1ull);
+    for (int jj0 = 0; jj0 < 64; jj0 += CELLS) {
+        if (!((live >> jj0) & gmask)) continue;
+        float vv[CELLS][RR];
+#pragma unroll
+        for (int u = 0; u < CELLS; ++u) {
+            const int64_t cell = j0 + jj0 + u < n_kv ? j0 + jj0 + u : n_kv - 1;
+            const char * vrow = vbase + cell * v_nb1;
+#pragma unroll
+            for (int r = 0; r < RR; ++r) {
+                const int dcol = lane + 64 * r;
+                vv[u][r] = kv_ld<VT>(vrow, dcol < DV ? dcol : DV - 1);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < CELLS; ++u) {
+            const float pj = __shfl(p, jj0 + u, 64);
+#pragma unroll
+            for (int r = 0; r < RR; ++r) acc[r] = fmaf(pj, vv[u][r], acc[r]);
+        }
+    }
+}
+
 template <int KT, int VT>
 __global__ void __launch_bounds__(256) k_attn_f32_rows(const tdesc q, const tdesc k, const tdesc v, const tdesc mask, const int has_mask, const float * __restrict__ sinks,
                                                        const tdesc dst, const float scale) {
@@ -85,18 +113,10 @@ __global__ void __launch_bounds__(256) k_attn_f32_rows(const tdesc q, const tdes
         m = m_new;
 #pragma unroll
         for (int r = 0; r < ATTN_F32_MAX_D / 64; ++r) acc[r] *= corr;
-        uint64_t todo = live;
-        while (todo) {
-            const int jj = __builtin_ctzll(todo);
-            todo &= todo - 1;
-            const float pj = __shfl(p, jj, 64);
-            const char * vrow = vbase + (j0 + jj) * v.nb[1];
-#pragma unroll
-            for (int r = 0; r < ATTN_F32_MAX_D / 64; ++r) {
-                const int dcol = lane + 64 * r;
-                if (dcol < DV) acc[r] = fmaf(pj, kv_ld<VT>(vrow, dcol), acc[r]);
-            }
-        }
+        // the visible cells' value rows, CELLS at a time with all their loads in flight together: a wave pays one trip to memory per group (measured: 2 us
+        // on an otherwise idle chip), so the groups are as large as the registers allow — 32 cells for value sizes up to 128, 16 beyond
+        if (DV <= 128) attn_f32_pv<VT, 32, 2>(p, live, vbase, v.nb[1], j0, n_kv, DV, lane, acc);
+        else attn_f32_pv<VT, 16, 4>(p, live, vbase, v.nb[1], j0, n_kv, DV, lane, acc);
     }
     if (lane == 0) { part_m[wave] = m; part_l[wave] = l; }
 #pragma unroll
