@@ -251,10 +251,10 @@ def attention_case(backend, H, kv_type, n_q, n_kv, heads, kv_heads, dk, dv, chun
 
 @pytest.mark.parametrize("kv_type", [L.F32, L.BF16])
 @pytest.mark.parametrize("n_q,n_kv,heads,kv_heads,dk,dv,chunk,sink", [
-    (1, 700, 4, 2, 64, 48, 0, True),      # one decoded token over 700 cells
+    (1, 700, 4, 2, 64, 40, 0, True),      # one decoded token over 700 cells
     (1, 300, 6, 2, 24, 136, 64, True),    # value rows wider than 128
     (5, 200, 2, 2, 16, 16, 7, False),     # a few tokens, tiny chunks, the plain soft-max
-    (70, 333, 4, 1, 64, 48, 50, True),    # a prompt portion (the tile form), chunk edges inside the portion
+    (70, 333, 4, 1, 64, 40, 50, True),    # a prompt portion (the tile form), chunk edges inside the portion
     (128, 640, 2, 2, 128, 128, 0, True),  # head size 128 both ways
     (33, 100, 3, 3, 40, 72, 9, False),
 ])
