@@ -410,3 +410,66 @@ def test_trace_run_command_line(tmp_path):
     r2 = np.fromfile(os.path.join(out_dir, "2.f32"), dtype="<f4").reshape(2, -1)
     assert row_err(r0, ref[[0, 8]]).max() <= F32_GATE
     assert row_err(r2, np.stack([ref[20], ref[1]])).max() <= F32_GATE  # request y repeats x's first tokens in its own slot
+
+
+def random_config(seed):
+    """a configuration drawn at random: widths with and without whole groups of 8 values, 1 - 6 layers, every chunk / rotary / feed-forward combination, value rows of one
+    total width (what value mixing needs) split over 1 - 8 key/value heads"""
+    rng = np.random.default_rng(seed)
+    width = int(rng.choice([32, 48, 64, 72, 96, 100, 128, 160, 36]))
+    vocab = int(rng.integers(40, 300))
+    kvd = int(rng.choice([24, 48, 96, 64, 40]))
+    layers = []
+    for _ in range(int(rng.integers(1, 7))):
+        opts = [(g, kvd // g) for g in (1, 2, 3, 4, 6, 8) if kvd % g == 0 and kvd // g >= 4]
+        G, dv = opts[int(rng.integers(len(opts)))]
+        H = G * int(rng.choice([1, 1, 2, 3, 4]))
+        dk = int(rng.choice([8, 12, 16, 24, 32, 40, 64, 96, 128, 20]))
+        rot = min(int(rng.choice([0, 2, 4, dk, 8])), dk) // 2 * 2
+        chunk = int(rng.choice([0, 3, 5, 16, 33, 64, 100, 257]))
+        kind = int(rng.integers(0, 4))
+        if kind == 0:
+            mlp = None
+        elif kind == 1:
+            mlp = ("dense", int(rng.choice([16, 40, 64, 100, 256])))
+        else:
+            ne = int(rng.integers(1, 9))
+            mlp = ("moe", int(rng.choice([8, 16, 24, 64])), ne, int(rng.integers(1, ne + 1)))
+        layers.append(dict(heads=H, kv_heads=G, dim=dk, vdim=dv, rot_dims=rot, rot_base=float(rng.choice([100.0, 10000.0, 1e6])), scale=float(rng.choice([dk ** -0.5, 0.1, 0.25])),
+                           chunk=chunk, v_mix=bool(rng.integers(0, 2)), mlp=mlp))
+    cfg = R.make_config(width, vocab, layers, eps=float(rng.choice([1e-6, 1e-5, 1e-3])), embed_scale=float(rng.choice([0.5, 1.0, 3.0])))
+    return cfg, rng
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_configurations(backend, tmp_path, seed):
+    """f32 serving of a random configuration: a whole prompt, then the same prompt in random portions beside a second request, its last tokens one by one"""
+    cfg, rng = random_config(seed)
+    W = R.random_weights(cfg, seed)
+    R.write_model(str(tmp_path), cfg, W)
+    n, n2 = int(rng.integers(60, 250)), int(rng.integers(5, 70))
+    t, t2 = rng.integers(0, cfg["vocab"], n).tolist(), rng.integers(0, cfg["vocab"], n2).tolist()
+    ref, ref2 = R.forward(cfg, W, t), R.forward(cfg, W, t2)
+    s = TraceSession(str(tmp_path), "float32", max_tokens=512, n_ubatch=128, backend=backend)
+    rows = s.step([{"id": "w", "tokens": t, "want": list(range(n))}], ["w"])
+    assert row_err(rows, ref).max() <= F32_GATE
+    got, got2, at, at2 = [], [], 0, 0
+    while at < n - 10:
+        c = min(int(rng.integers(1, 70)), n - 10 - at)
+        ent = [{"id": "a", "tokens": t[at:at + c], "want": list(range(c))}]
+        c2 = min(int(rng.integers(1, 20)), n2 - at2)
+        if c2 > 0:
+            ent.append({"id": "b", "tokens": t2[at2:at2 + c2], "want": list(range(c2))})
+        r = s.step(ent, [])
+        got.append(r[:c])
+        if c2 > 0:
+            got2.append(r[c:c + c2])
+        at, at2 = at + c, at2 + max(c2, 0)
+    while at < n:
+        got.append(s.step([{"id": "a", "tokens": [t[at]], "want": [0]}], []))
+        at += 1
+    s.step([], ["a", "b"])
+    assert row_err(np.concatenate(got), ref).max() <= F32_GATE
+    if got2:
+        assert row_err(np.concatenate(got2), ref2[:at2]).max() <= F32_GATE
+    s.close()
