@@ -34,13 +34,17 @@ __device__ __forceinline__ float wave_sum_f(float v) {
     return v;
 }
 
-constexpr int ATTN_F32_MAX_D = 256;   // largest head size (query/key or value)
+constexpr int ATTN_F32_MAX_D = 640;   // largest head size (query/key or value): a latent cache row (latent + rotated part) serves as the key of every head
 constexpr float ATTN_F32_LOW = -1e30f;  // "no score yet": finite, so that differences of maxima never give NaN
 
 // mask element -> additive term (f16 or f32 mask rows; -inf hides the cell)
 __device__ __forceinline__ float mask_ld(const char * __restrict__ mrow, const int mtype, const int64_t j) {
     return mtype == GGML_TYPE_F16 ? h2f(((const uint16_t *) mrow)[j]) : ((const float *) mrow)[j];
 }
+
+// the additive term of a visible cell: the mask's value itself, or — with a per-head distance penalty (r1, r2) — the mask's value read as the distance
+// between query and cell: -r1 ln(1 + r2 distance)
+__device__ __forceinline__ float mask_term(const float mv, const bool pen, const float r1, const float r2) { return pen ? -r1 * logf(1.0f + r2 * mv) : mv; }
 
 // acc[r] += sum over the block's visible cells of p[cell] * V[cell][lane + 64 r]: no branches around the loads (a lane beyond the row's end re-reads the last
 // column, its sum is dropped later; hidden cells enter with weight 0)
@@ -72,7 +76,7 @@ __device__ __forceinline__ void attn_f32_pv(const float p, const uint64_t live, 
 
 template <int KT, int VT>
 __global__ void __launch_bounds__(256) k_attn_f32_rows(const tdesc q, const tdesc k, const tdesc v, const tdesc mask, const int has_mask, const float * __restrict__ sinks,
-                                                       const tdesc dst, const float scale) {
+                                                       const float * __restrict__ r12, const tdesc dst, const float scale) {
     __shared__ float qs[ATTN_F32_MAX_D];
     __shared__ float part_acc[4][ATTN_F32_MAX_D];
     __shared__ float part_m[4], part_l[4];
@@ -87,6 +91,8 @@ __global__ void __launch_bounds__(256) k_attn_f32_rows(const tdesc q, const tdes
     const char * mrow = has_mask ? mask.data + t * mask.nb[1] : nullptr;
     const char * kbase = k.data + g * k.nb[2];
     const char * vbase = v.data + g * v.nb[2];
+    const bool pen = r12 != nullptr;
+    const float r1 = pen ? r12[h] : 0.0f, r2 = pen ? r12[q.ne[2] + h] : 0.0f;
     float m = ATTN_F32_LOW, l = 0.0f;
     if (sinks && wave == 0) { m = sinks[h]; l = 1.0f; }  // the sink: exp(sink - m) = 1 in the denominator, nothing in the numerator
     float acc[ATTN_F32_MAX_D / 64];
@@ -104,7 +110,7 @@ __global__ void __launch_bounds__(256) k_attn_f32_rows(const tdesc q, const tdes
             const char * krow = kbase + j * k.nb[1];
             float d = 0.0f;
             for (int i = 0; i < DK; ++i) d = fmaf(qs[i], kv_ld<KT>(krow, i), d);
-            s = d * scale + mv;
+            s = d * scale + mask_term(mv, pen, r1, r2);
         }
         const float m_new = fmaxf(m, wave_max_f(s));
         const float p = vis ? expf(s - m_new) : 0.0f;
@@ -116,7 +122,8 @@ __global__ void __launch_bounds__(256) k_attn_f32_rows(const tdesc q, const tdes
         // the visible cells' value rows, CELLS at a time with all their loads in flight together: a wave pays one trip to memory per group (measured: 2 us
         // on an otherwise idle chip), so the groups are as large as the registers allow — 32 cells for value sizes up to 128, 16 beyond
         if (DV <= 128) attn_f32_pv<VT, 32, 2>(p, live, vbase, v.nb[1], j0, n_kv, DV, lane, acc);
-        else attn_f32_pv<VT, 16, 4>(p, live, vbase, v.nb[1], j0, n_kv, DV, lane, acc);
+        else if (DV <= 256) attn_f32_pv<VT, 16, 4>(p, live, vbase, v.nb[1], j0, n_kv, DV, lane, acc);
+        else attn_f32_pv<VT, 8, ATTN_F32_MAX_D / 64>(p, live, vbase, v.nb[1], j0, n_kv, DV, lane, acc);
     }
     if (lane == 0) { part_m[wave] = m; part_l[wave] = l; }
 #pragma unroll
@@ -141,8 +148,8 @@ __global__ void __launch_bounds__(256) k_attn_f32_rows(const tdesc q, const tdes
 
 // prompt batches: 64 query tokens x one head per workgroup; K / V blocks of 64 cells staged in LDS as f32
 template <int KT, int VT, int DKP, int DVP>   // DKP / DVP: head sizes rounded up to a multiple of 32 / 64 (LDS row lengths)
-__global__ void __launch_bounds__(256) k_attn_f32_tile(const tdesc q, const tdesc k, const tdesc v, const tdesc mask, const float * __restrict__ sinks, const tdesc dst,
-                                                       const float scale) {
+__global__ void __launch_bounds__(256) k_attn_f32_tile(const tdesc q, const tdesc k, const tdesc v, const tdesc mask, const float * __restrict__ sinks,
+                                                       const float * __restrict__ r12, const tdesc dst, const float scale) {
     constexpr int QT = 64, KB = 64, QW = QT / 4;  // queries per workgroup, cells per block, queries per wave
     constexpr int KS = DKP + 1;                   // K row stride in LDS (odd: lanes that read column i of 64 different rows hit 64 different banks)
     extern __shared__ float lds[];
@@ -157,6 +164,8 @@ __global__ void __launch_bounds__(256) k_attn_f32_tile(const tdesc q, const tdes
     const int64_t g = h / (q.ne[2] / k.ne[2]);
     const char * kbase = k.data + g * k.nb[2];
     const char * vbase = v.data + g * v.nb[2];
+    const bool pen = r12 != nullptr;
+    const float r1 = pen ? r12[h] : 0.0f, r2 = pen ? r12[q.ne[2] + h] : 0.0f;
     for (int e = threadIdx.x; e < QT * DKP; e += 256) {
         const int qi = e / DKP, i = e % DKP;
         const int64_t t = t0 + qi;
@@ -209,7 +218,7 @@ __global__ void __launch_bounds__(256) k_attn_f32_tile(const tdesc q, const tdes
             const float * qr = Qs + ql * DKP;
             const float * kr = Ks + lane * KS;
             for (int i = 0; i < DK; ++i) d = fmaf(qr[i], kr[i], d);
-            const float s = vis ? d * scale + mv : -INFINITY;
+            const float s = vis ? d * scale + mask_term(mv, pen, r1, r2) : -INFINITY;
             const float m_new = fmaxf(m[qi], wave_max_f(s));
             const float p = vis ? expf(s - m_new) : 0.0f;
             const float corr = expf(m[qi] - m_new);
@@ -258,7 +267,8 @@ __device__ __forceinline__ uint32_t att_bf16_bits(const float f) {
     return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
 }
 template <int DK16, int DVT>
-__global__ void __launch_bounds__(256) k_attn_mma_bf16(const tdesc q, const tdesc k, const tdesc v, const tdesc mask, const float * __restrict__ sinks, const tdesc dst, const float scale) {
+__global__ void __launch_bounds__(256) k_attn_mma_bf16(const tdesc q, const tdesc k, const tdesc v, const tdesc mask, const float * __restrict__ sinks, const float * __restrict__ r12, const tdesc dst,
+                                                       const float scale) {
     constexpr int VS = 36;  // V^T row stride in LDS (bf16 elements): 72 bytes keeps the 8-byte reads aligned and spreads the rows over the banks
     __shared__ __attribute__((aligned(16))) uint16_t Vt[DVT * 32 * VS];
     __shared__ int flag[2];
@@ -284,6 +294,8 @@ __global__ void __launch_bounds__(256) k_attn_mma_bf16(const tdesc q, const tdes
             qf[s] = make_uint4(b[0] | (b[1] << 16), b[2] | (b[3] << 16), b[4] | (b[5] << 16), b[6] | (b[7] << 16));
         }
     }
+    const bool pen = r12 != nullptr;
+    const float r1 = pen ? r12[h] : 0.0f, r2 = pen ? r12[q.ne[2] + h] : 0.0f;
     float m = sinks ? sinks[h] : ATTN_F32_LOW, l = sinks ? 1.0f : 0.0f;
     att_f16v O[DVT];
 #pragma unroll
@@ -362,7 +374,7 @@ __global__ void __launch_bounds__(256) k_attn_mma_bf16(const tdesc q, const tdes
         float mx = ATTN_F32_LOW;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            S[i] = mv[i] > -INFINITY ? S[i] * scale + mv[i] : -INFINITY;
+            S[i] = mv[i] > -INFINITY ? S[i] * scale + mask_term(mv[i], pen, r1, r2) : -INFINITY;
             mx = fmaxf(mx, S[i]);
         }
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
@@ -436,7 +448,7 @@ bool attn_f32_applies(const tdesc & q, const tdesc & k, const tdesc & v, const t
 }
 
 template <int KT, int VT>
-static void attn_f32_launch_t(hipStream_t s, const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const float * sinks, const tdesc & dst, float scale) {
+static void attn_f32_launch_t(hipStream_t s, const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const float * sinks, const float * r12, const tdesc & dst, float scale) {
     const int64_t n_q = q.ne[1], H = q.ne[2];
     const int DK = (int) q.ne[0], DV = (int) v.ne[0];
     if constexpr (KT == GGML_TYPE_BF16 && VT == GGML_TYPE_BF16) {
@@ -451,7 +463,7 @@ static void attn_f32_launch_t(hipStream_t s, const tdesc & q, const tdesc & k, c
             const dim3 grid((unsigned) ((n_q + 32 * nw - 1) / (32 * nw)), (unsigned) H);
             const dim3 block((unsigned) (64 * nw));
             const int dk16 = (DK + 15) / 16, dvt = (DV + 31) / 32;
-#define MI_ATT_MMA(A, B) hipLaunchKernelGGL((k_attn_mma_bf16<A, B>), grid, block, 0, s, q, k, v, *mask, sinks, dst, scale)
+#define MI_ATT_MMA(A, B) hipLaunchKernelGGL((k_attn_mma_bf16<A, B>), grid, block, 0, s, q, k, v, *mask, sinks, r12, dst, scale)
             const int a = dk16 <= 2 ? 2 : (dk16 <= 4 ? 4 : 8), b = dvt <= 1 ? 1 : (dvt <= 2 ? 2 : 4);
             if (a == 2 && b == 1) MI_ATT_MMA(2, 1); else if (a == 2 && b == 2) MI_ATT_MMA(2, 2); else if (a == 2) MI_ATT_MMA(2, 4);
             else if (a == 4 && b == 1) MI_ATT_MMA(4, 1); else if (a == 4 && b == 2) MI_ATT_MMA(4, 2); else if (a == 4) MI_ATT_MMA(4, 4);
@@ -467,7 +479,7 @@ static void attn_f32_launch_t(hipStream_t s, const tdesc & q, const tdesc & k, c
             const size_t lds = ((size_t) 64 * (dkp + 1) + (size_t) 64 * dvp + (size_t) 64 * dkp) * sizeof(float);
             // (more than the 64 KB a kernel gets by default: up to 97 KB of the CU's 160 KB; the attribute is per device and cheap to set again)
             if (lds > 48 * 1024) (void) hipFuncSetAttribute((const void *) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds);
-            hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, q, k, v, *mask, sinks, dst, scale);
+            hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, q, k, v, *mask, sinks, r12, dst, scale);
         };
         const bool k64 = DK <= 64, v64 = DV <= 64;
         if (k64 && v64) go(k_attn_f32_tile<KT, VT, 64, 64>, 64, 64);
@@ -476,12 +488,12 @@ static void attn_f32_launch_t(hipStream_t s, const tdesc & q, const tdesc & k, c
         else go(k_attn_f32_tile<KT, VT, 128, 128>, 128, 128);
         return;
     }
-    hipLaunchKernelGGL((k_attn_f32_rows<KT, VT>), dim3((unsigned) n_q, (unsigned) H), dim3(256), 0, s, q, k, v, mask ? *mask : q, mask ? 1 : 0, sinks, dst, scale);
+    hipLaunchKernelGGL((k_attn_f32_rows<KT, VT>), dim3((unsigned) n_q, (unsigned) H), dim3(256), 0, s, q, k, v, mask ? *mask : q, mask ? 1 : 0, sinks, r12, dst, scale);
 }
 
-void launch_attn_f32(hipStream_t s, const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const float * sinks, const tdesc & dst, float scale) {
+void launch_attn_f32(hipStream_t s, const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const float * sinks, const float * r12, const tdesc & dst, float scale) {
     if (q.ne[1] == 0 || q.ne[2] == 0) return;
-#define MI_ATTN_F32_CASE(KT, VT) if (k.type == KT && v.type == VT) { attn_f32_launch_t<KT, VT>(s, q, k, v, mask, sinks, dst, scale); return; }
+#define MI_ATTN_F32_CASE(KT, VT) if (k.type == KT && v.type == VT) { attn_f32_launch_t<KT, VT>(s, q, k, v, mask, sinks, r12, dst, scale); return; }
     MI_ATTN_F32_CASE(GGML_TYPE_F32, GGML_TYPE_F32)
     MI_ATTN_F32_CASE(GGML_TYPE_BF16, GGML_TYPE_BF16)
     MI_ATTN_F32_CASE(GGML_TYPE_F16, GGML_TYPE_F16)

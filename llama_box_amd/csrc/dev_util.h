@@ -176,6 +176,13 @@ __device__ __forceinline__ void rope_cos_sin_exact(const int ip, const float pos
     cs = cosf(theta);
     sn = sinf(theta);
 }
+// the angle of pair ip as pos * freq[ip] with the pairs' frequencies given as a table (ROPE op_params[3] == 2: src[2] holds frequencies, not divisors); cos and sin
+// are multiplied by `mag`.  For frequency schedules that the host computes once (a blend of scaled and unscaled frequencies, for instance).
+__device__ __forceinline__ void rope_cos_sin_table(const int ip, const float pos_f, const float * __restrict__ freq, const float mag, float & cs, float & sn) {
+    const float theta = pos_f * freq[ip];
+    cs = cosf(theta) * mag;
+    sn = sinf(theta) * mag;
+}
 __device__ __forceinline__ void rope_cos_sin(const int ip, const float pos_f, const float * __restrict__ ff, const rope_consts rc, float & cs, float & sn) {
     float theta = pos_f;
     for (int k = 0; k < ip; ++k) theta *= rc.theta_scale;

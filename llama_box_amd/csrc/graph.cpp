@@ -67,6 +67,8 @@ static bool fa_f32_route(const ggml_tensor * op) {
     const ggml_tensor * m = op->src[3];
     if (ggml_abi_op_param_f32(op, 1) != 0.0f || ggml_abi_op_param_f32(op, 2) != 0.0f) return false;  // no ALiBi slopes, no soft-capping there
     if (op->src[4] && (op->src[4]->type != GGML_TYPE_F32 || ggml_abi_nelements(op->src[4]) < a->ne[2])) return false;
+    // src[5]: (r1, r2) per head of a logarithmic distance penalty; the F32 mask then holds distances
+    if (op->src[5] && (op->src[5]->type != GGML_TYPE_F32 || !ggml_abi_is_contiguous(op->src[5]) || ggml_abi_nelements(op->src[5]) != 2 * a->ne[2] || !m || m->type != GGML_TYPE_F32)) return false;
     const tdesc md = m ? TD(m) : TD(a);
     return attn_f32_applies(TD(a), TD(k), TD(v), m ? &md : nullptr, TD(op));
 }
@@ -85,6 +87,7 @@ static int fa_route(const ggml_tensor * op) {
         (void) wide_k; (void) wide_v;
         if (plain && (f32_mask || odd_shape) && fa_f32_route(op)) return 4;
     }
+    if (op->src[5]) return 0;  // (the distance penalty is a feature of the 32-bit kernels alone)
     if (k->type == GGML_TYPE_Q8_0 && v->type == GGML_TYPE_Q8_0) {
         // quantised KV cache: served by the lane-parallel kernel (head_dim 128, 1 .. 8 query heads per KV head, no soft-capping / ALiBi)
         const int64_t g = k->ne[2] ? a->ne[2] / k->ne[2] : 0;
@@ -118,6 +121,8 @@ static bool bf16_rows_in_blocks(const ggml_tensor * a) { return (a->ne[0] % 32) 
 // ROPE op_params[3] (ggml's unused n_ctx slot) == 1: the graph asks for per-pair frequencies computed on their own (dev_util.h: rope_cos_sin_exact); honoured for the
 // plain case only (no frequency scaling, no YaRN, no factors, not multi-section)
 static int rope_exact_freq(const ggml_tensor * n) {
+    // == 2: src[2] is a table of the pairs' frequencies themselves (dev_util.h: rope_cos_sin_table)
+    if (n->op_params[3] == 2 && n->src[2] && !(n->op_params[2] & GGML_ROPE_TYPE_MROPE)) return 2;
     return (n->op_params[3] == 1 && !n->src[2] && !(n->op_params[2] & GGML_ROPE_TYPE_MROPE) && ggml_abi_op_param_f32(n, 6) == 1.0f && ggml_abi_op_param_f32(n, 7) == 0.0f &&
             ggml_abi_op_param_f32(n, 8) == 1.0f) ? 1 : 0;
 }
@@ -150,6 +155,8 @@ bool supports_op(const ggml_tensor * op) {
             return a->type == GGML_TYPE_F32 && b->type == GGML_TYPE_F32 && op->type == GGML_TYPE_F32;
         case GGML_OP_SCALE:
             return is_f32_contig(a) && is_f32_contig(op);
+        case GGML_OP_CONCAT:
+            return a->type == GGML_TYPE_F32 && b && b->type == GGML_TYPE_F32 && op->type == GGML_TYPE_F32 && op->op_params[0] >= 0 && op->op_params[0] < 4;
         case GGML_OP_RMS_NORM:
         case GGML_OP_NORM:
             return a->type == GGML_TYPE_F32 && a->nb[0] == 4 && op->nb[0] == 4;
@@ -2043,6 +2050,12 @@ static int run_node(exec_state & st, int i) {
             c->st.kernel_launches++;
             return 1;
         }
+        case GGML_OP_CONCAT: {
+            timed_scope ts(c, "concat", (double) ggml_abi_nbytes(n) * 2);
+            launch_concat(s, TD(a), TD(b), TD(n), n->op_params[0]);
+            c->st.kernel_launches++;
+            return 1;
+        }
         case GGML_OP_SCALE: {
             // SCALE(x, a), SCALE(y, b), ADD of the two (a blend of two tensors): one pass
             ggml_tensor * s2 = next(1), * ad = next(2);
@@ -2266,7 +2279,7 @@ static int run_node(exec_state & st, int i) {
                         }
                         if (clean) { cast = t; cast_at = k; }
                     }
-                    if (!rope && t->op == GGML_OP_ROPE && t->type == GGML_TYPE_F32 && !(t->op_params[2] & GGML_ROPE_TYPE_MROPE) && t->src[1] && t->src[1]->op == GGML_OP_NONE &&
+                    if (!rope && t->op == GGML_OP_ROPE && t->type == GGML_TYPE_F32 && t->op_params[3] == 0 && !(t->op_params[2] & GGML_ROPE_TYPE_MROPE) && t->src[1] && t->src[1]->op == GGML_OP_NONE &&
                         t->src[1]->type == GGML_TYPE_I32 && (!t->src[2] || t->src[2]->op == GGML_OP_NONE))
                         rope = t;
                 }
@@ -2400,7 +2413,7 @@ static int run_node(exec_state & st, int i) {
                     p.exact_freq = rope_exact_freq(n);
                     const ggml_tensor * sr = g->nodes[ks];
                     timed_scope ts(c, "rope_store_rows", (double) ggml_abi_nbytes(n) * 2);
-                    launch_rope_store(s, TD(a), TD(b), (const int64_t *) sr->src[1]->data, TD(sr), p);
+                    launch_rope_store(s, TD(a), TD(b), nullptr, (const int64_t *) sr->src[1]->data, TD(sr), p);
                     c->st.kernel_launches++;
                     c->st.fused_nodes++;
                     mark_done(st, ks);
@@ -2437,7 +2450,7 @@ static int run_node(exec_state & st, int i) {
             if (fa_route(n) == 4) {
                 const tdesc md4 = m ? TD(m) : qd;
                 timed_scope ts(c, "attn_f32", (double) ggml_abi_nbytes(k) + (double) ggml_abi_nbytes(v));
-                launch_attn_f32(s, qd, kd, vd, m ? &md4 : nullptr, n->src[4] ? (const float *) n->src[4]->data : nullptr, TD(n), p.scale);
+                launch_attn_f32(s, qd, kd, vd, m ? &md4 : nullptr, n->src[4] ? (const float *) n->src[4]->data : nullptr, n->src[5] ? (const float *) n->src[5]->data : nullptr, TD(n), p.scale);
                 c->st.kernel_launches++;
                 c->st.attn_f32_nodes++;
                 return 1;

@@ -170,7 +170,9 @@ size_t mul_mat_id_workspace_bytes(const tdesc & as, const tdesc & ids);
 bool launch_mul_mat_id(hipStream_t s, const tdesc & as, const tdesc & b, const tdesc & ids, const tdesc & d, void * ws, size_t ws_bytes, bool lists_valid);  // true: the batched form ran and left the lists in ws
 // FLASH_ATTN_EXT in 32-bit arithmetic over f32 / bf16 / f16 K and V read in place, any head sizes up to 256, K and V sizes independent (attn_f32.hip)
 bool attn_f32_applies(const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const tdesc & dst);
-void launch_attn_f32(hipStream_t s, const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const float * sinks, const tdesc & dst, float scale);
+// r12 (optional: r1 of every head, then r2 of every head): the mask then holds the DISTANCE between query and cell for visible pairs (-inf for hidden ones) and the score is
+// q.k * scale - r1 ln(1 + r2 distance)
+void launch_attn_f32(hipStream_t s, const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const float * sinks, const float * r12, const tdesc & dst, float scale);
 // ---- non-flash attention chain of a small batch over position lists (attn_nf.hip)
 size_t attn_nf_list_scratch_bytes(const tdesc & q, const tdesc & k, int * dq_out);
 bool launch_attn_nf_list(hipStream_t s, const tdesc & q, const tdesc & k, const tdesc & v, const tdesc & mask, const tdesc & dst, const int * lists, int list_stride,
@@ -248,6 +250,7 @@ void launch_splitk_rms_norm_mul_quantize(hipStream_t s, const splitk_src & sk, i
 void launch_rms_norm_mul_quantize(hipStream_t s, const tdesc & x, const float * w, float eps, void * dst_q8k);
 void launch_swiglu_quantize(hipStream_t s, const tdesc & a, const tdesc * b, int64_t nc, int swapped, void * dst_q8k);
 void launch_cpy(hipStream_t s, const tdesc & src, const tdesc & dst);
+void launch_concat(hipStream_t s, const tdesc & a, const tdesc & b, const tdesc & dst, int dim);  // f32, any strides
 void launch_get_rows(hipStream_t s, const tdesc & src, const tdesc & idx, const tdesc & dst);
 void launch_set_rows(hipStream_t s, const tdesc & src, const tdesc & idx, const tdesc & dst);
 void launch_cpy_q8_0(hipStream_t s, const void * src, void * dst, int64_t n_values, bool to_q8);  // contiguous Q8_0 <-> F32 (K-shift of a quantised cache)
@@ -277,7 +280,7 @@ struct rope_params {
     int n_dims, mode, n_ctx_orig;
     float freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow;
     int sections[4];  // ggml_rope_multi (mode & GGML_ROPE_TYPE_MROPE): pairs per position stream (time, height, width, extra)
-    int exact_freq = 0;  // 1: every pair's frequency base^(-2 i / n_dims) is computed on its own (f64, rounded once) instead of by the recurrence theta *= theta_scale
+    int exact_freq = 0;  // 2: the frequency of every pair is read from a table (src[2] of the op) and cos / sin are multiplied by attn_factor; 1: every pair's frequency base^(-2 i / n_dims) is computed on its own (f64, rounded once) instead of by the recurrence theta *= theta_scale
 };
 void rope_host_consts(const rope_params & p, float & theta_scale, float & corr0, float & corr1);
 // (cos, sin) of every (token, rotation pair) of a small batch — rope_cos_sin's arithmetic, once per graph run instead of once per layer and element
@@ -309,7 +312,7 @@ bool rope_qk_store_vec_ok(const rope_store_args & a, int n_tokens);
 void launch_rope_qk_store_vec(hipStream_t s, const rope_store_args & a, int n_tokens, const float * tab);
 void launch_rope(hipStream_t s, const tdesc & src, const tdesc & pos, const float * freq_factors, const tdesc & dst, const rope_params & p);
 // ROPE (no frequency factors) + SET_ROWS into a cache kept in f32 / f16 / bf16, and a x + b y + SET_ROWS: the value goes straight into cache row idx[t]
-void launch_rope_store(hipStream_t s, const tdesc & src /* [D, heads, T] f32 */, const tdesc & pos, const int64_t * idx, const tdesc & cache, const rope_params & p);
+void launch_rope_store(hipStream_t s, const tdesc & src /* [D, heads, T] f32 */, const tdesc & pos, const float * freq /* exact_freq == 2 */, const int64_t * idx, const tdesc & cache, const rope_params & p);
 void launch_axpby_store(hipStream_t s, const float * x, float a, const float * y, float b, int64_t n, int64_t n_tok, const int64_t * idx, const tdesc & cache);
 void launch_soft_max(hipStream_t s, const tdesc & src, const tdesc * mask, const float * sinks, const tdesc & dst, float scale, float max_bias);
 

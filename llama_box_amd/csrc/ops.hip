@@ -518,6 +518,31 @@ void launch_cpy(hipStream_t s, const tdesc & a, const tdesc & d) {
     else { MI_ERR("launch_cpy: unsupported types %d -> %d", st, dt); abort(); }
 }
 
+// CONCAT: d = a and b joined along dimension `dim` (f32, any strides): one element per thread step, the source chosen by the index along dim
+__global__ void __launch_bounds__(256) k_concat(const tdesc a, const tdesc b, const tdesc d, const int dim, const int64_t n) {
+    for (int64_t e = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t) gridDim.x * blockDim.x) {
+        int64_t r = e, ix[4];
+        ix[0] = r % d.ne[0]; r /= d.ne[0];
+        ix[1] = r % d.ne[1]; r /= d.ne[1];
+        ix[2] = r % d.ne[2]; r /= d.ne[2];
+        ix[3] = r;
+        char * out = d.data + ix[0] * d.nb[0] + ix[1] * d.nb[1] + ix[2] * d.nb[2] + ix[3] * d.nb[3];
+        const int64_t na = dim == 0 ? a.ne[0] : dim == 1 ? a.ne[1] : dim == 2 ? a.ne[2] : a.ne[3];
+        const int64_t at = dim == 0 ? ix[0] : dim == 1 ? ix[1] : dim == 2 ? ix[2] : ix[3];
+        const bool first = at < na;
+        const int64_t sh = first ? 0 : na;
+        const int64_t s0 = ix[0] - (dim == 0 ? sh : 0), s1 = ix[1] - (dim == 1 ? sh : 0), s2 = ix[2] - (dim == 2 ? sh : 0), s3 = ix[3] - (dim == 3 ? sh : 0);
+        const tdesc & src = first ? a : b;
+        *(float *) out = *(const float *) (src.data + s0 * src.nb[0] + s1 * src.nb[1] + s2 * src.nb[2] + s3 * src.nb[3]);
+    }
+}
+void launch_concat(hipStream_t s, const tdesc & a, const tdesc & b, const tdesc & d, int dim) {
+    const int64_t n = d.ne[0] * d.ne[1] * d.ne[2] * d.ne[3];
+    if (n == 0) return;
+    const unsigned grid = (unsigned) std::min<int64_t>((n + 255) / 256, 8192);
+    hipLaunchKernelGGL(k_concat, dim3(grid), dim3(256), 0, s, a, b, d, dim, n);
+}
+
 // ------------------------------------------------------------------------------------------------ GET_ROWS
 // dequantize_row_{q8_0,q4_K,q5_K,q6_K} element formulas: one workgroup per gathered row
 __device__ __forceinline__ void k4_scale_min(int j, const uint8_t * q, int & sc, int & m) {
@@ -681,7 +706,8 @@ template <bool F16IO> __global__ void __launch_bounds__(64) k_rope(const tdesc a
         if (F16IO) { x0 = h2f(((const uint16_t *) src)[ia]); x1 = h2f(((const uint16_t *) src)[ib]); }
         else { x0 = ((const float *) src)[ia]; x1 = ((const float *) src)[ib]; }
         float cs, sn;
-        if (p.exact_freq) rope_cos_sin_exact(ip, pos_f, p.freq_base, p.n_dims, cs, sn);
+        if (p.exact_freq == 2) rope_cos_sin_table(ip, pos_f, ff, p.attn_factor, cs, sn);
+        else if (p.exact_freq) rope_cos_sin_exact(ip, pos_f, p.freq_base, p.n_dims, cs, sn);
         else rope_cos_sin(ip, pos_f, ff, rope_consts{theta_scale, p.freq_scale, p.ext_factor, p.attn_factor, corr0, corr1}, cs, sn);
         if (F16IO) {
             ((uint16_t *) dst)[ia] = f2h(x0 * cs - x1 * sn);
@@ -1038,7 +1064,7 @@ __device__ __forceinline__ void store_as(char * __restrict__ row, const int type
     else if (type == GGML_TYPE_BF16) ((uint16_t *) row)[i] = f2bf(v);
     else ((uint16_t *) row)[i] = f2h(v);
 }
-__global__ void __launch_bounds__(64) k_rope_store(const tdesc a, const tdesc pos, const int64_t * __restrict__ idx, char * __restrict__ cache, const int64_t cache_nb1, const int cache_type,
+__global__ void __launch_bounds__(64) k_rope_store(const tdesc a, const tdesc pos, const float * __restrict__ ff, const int64_t * __restrict__ idx, char * __restrict__ cache, const int64_t cache_nb1, const int cache_type,
                                                    const rope_params p, const float theta_scale, const float corr0, const float corr1) {
     const int64_t i1 = blockIdx.x, i2 = blockIdx.y;
     const int n_pairs = p.n_dims / 2;
@@ -1051,18 +1077,19 @@ __global__ void __launch_bounds__(64) k_rope_store(const tdesc a, const tdesc po
         const int ia = neox ? ip : 2 * ip, ib = neox ? ip + n_pairs : 2 * ip + 1;
         const float x0 = src[ia], x1 = src[ib];
         float cs, sn;
-        if (p.exact_freq) rope_cos_sin_exact(ip, pos_f, p.freq_base, p.n_dims, cs, sn);
+        if (p.exact_freq == 2) rope_cos_sin_table(ip, pos_f, ff, p.attn_factor, cs, sn);
+        else if (p.exact_freq) rope_cos_sin_exact(ip, pos_f, p.freq_base, p.n_dims, cs, sn);
         else rope_cos_sin(ip, pos_f, nullptr, rope_consts{theta_scale, p.freq_scale, p.ext_factor, p.attn_factor, corr0, corr1}, cs, sn);
         store_as(row, cache_type, base + ia, x0 * cs - x1 * sn);
         store_as(row, cache_type, base + ib, x0 * sn + x1 * cs);
     }
     for (int64_t i0 = p.n_dims + threadIdx.x; i0 < a.ne[0]; i0 += blockDim.x) store_as(row, cache_type, base + i0, src[i0]);
 }
-void launch_rope_store(hipStream_t s, const tdesc & a, const tdesc & pos, const int64_t * idx, const tdesc & cache, const rope_params & p) {
+void launch_rope_store(hipStream_t s, const tdesc & a, const tdesc & pos, const float * ff, const int64_t * idx, const tdesc & cache, const rope_params & p) {
     if (a.ne[1] * a.ne[2] == 0) return;
     float theta_scale, c0, c1;
     rope_host_consts(p, theta_scale, c0, c1);
-    hipLaunchKernelGGL(k_rope_store, dim3((unsigned) a.ne[1], (unsigned) a.ne[2]), dim3(64), 0, s, a, pos, idx, cache.data, cache.nb[1], cache.type, p, theta_scale, c0, c1);
+    hipLaunchKernelGGL(k_rope_store, dim3((unsigned) a.ne[1], (unsigned) a.ne[2]), dim3(64), 0, s, a, pos, ff, idx, cache.data, cache.nb[1], cache.type, p, theta_scale, c0, c1);
 }
 // a x + b y (k_axpby's arithmetic) stored as rows of a cache: row t of n values goes to cache row idx[t]
 __global__ void __launch_bounds__(256) k_axpby_store(const float * __restrict__ x, const float a, const float * __restrict__ y, const float b, const int64_t n, const int64_t * __restrict__ idx,

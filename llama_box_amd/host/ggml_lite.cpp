@@ -400,6 +400,22 @@ struct ggml_tensor * ggml_mul_mat(struct ggml_context * ctx, struct ggml_tensor 
 }
 void ggml_mul_mat_set_prec(struct ggml_tensor * a, enum ggml_prec prec) { a->op_params[0] = (int32_t) prec; }
 
+// a and b joined along dimension `dim` (the other dimensions equal)
+struct ggml_tensor * ggml_concat(struct ggml_context * ctx, struct ggml_tensor * a, struct ggml_tensor * b, int dim) {
+    LITE_ASSERT(dim >= 0 && dim < 4 && a->type == b->type);
+    int64_t ne[4];
+    for (int d = 0; d < 4; ++d) {
+        if (d == dim) { ne[d] = a->ne[d] + b->ne[d]; continue; }
+        LITE_ASSERT(a->ne[d] == b->ne[d]);
+        ne[d] = a->ne[d];
+    }
+    ggml_tensor * r = ggml_new_tensor(ctx, a->type, 4, ne);
+    r->op_params[0] = dim;
+    r->op = GGML_OP_CONCAT;
+    r->src[0] = a;
+    r->src[1] = b;
+    return r;
+}
 struct ggml_tensor * ggml_get_rows(struct ggml_context * ctx, struct ggml_tensor * a, struct ggml_tensor * b) {
     LITE_ASSERT(a->ne[2] == b->ne[1] && b->ne[3] == 1 && b->type == GGML_TYPE_I32);
     const ggml_type type = a->type == GGML_TYPE_I32 ? GGML_TYPE_I32 : GGML_TYPE_F32;
@@ -550,6 +566,19 @@ struct ggml_tensor * ggml_flash_attn_ext(struct ggml_context * ctx, struct ggml_
 void ggml_rope_set_exact_freq(struct ggml_tensor * a) {
     LITE_ASSERT(a->op == GGML_OP_ROPE);
     a->op_params[3] = 1;
+}
+// harness extension: src[2] of the ROPE holds every pair's FREQUENCY (n_dims / 2 values: the angle is pos * c[i], one f32 product), and cos / sin are
+// multiplied by attn_factor — for frequency schedules computed once on the host (YaRN's blend, for instance): op_params[3] == 2
+void ggml_rope_set_freq_table(struct ggml_tensor * a) {
+    LITE_ASSERT(a->op == GGML_OP_ROPE && a->src[2] != nullptr);
+    a->op_params[3] = 2;
+}
+// harness extension: a per-head penalty on the distance between query and key, score -= r1[h] * ln(1 + r2[h] * distance).  `r12` is f32 [heads, 2]
+// (r1 of every head, then r2 of every head); the op's F32 mask then holds the DISTANCE of every visible (query, cell) pair (>= 0) and -inf for hidden ones: src[5]
+void ggml_flash_attn_ext_add_log_distance(struct ggml_tensor * a, struct ggml_tensor * r12) {
+    LITE_ASSERT(a->op == GGML_OP_FLASH_ATTN_EXT && a->src[3] != nullptr && a->src[3]->type == GGML_TYPE_F32);
+    LITE_ASSERT(r12->type == GGML_TYPE_F32 && r12->ne[0] == a->src[0]->ne[2] && r12->ne[1] == 2 && ggml_is_contiguous(r12));
+    a->src[5] = r12;
 }
 void ggml_flash_attn_ext_set_prec(struct ggml_tensor * a, enum ggml_prec prec) {
     LITE_ASSERT(a->op == GGML_OP_FLASH_ATTN_EXT);

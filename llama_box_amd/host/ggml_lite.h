@@ -85,6 +85,7 @@ struct ggml_tensor * ggml_top_k(struct ggml_context * ctx, struct ggml_tensor * 
 struct ggml_tensor * ggml_mul_mat_id(struct ggml_context * ctx, struct ggml_tensor * as, struct ggml_tensor * b, struct ggml_tensor * ids);
 struct ggml_tensor * ggml_mul_mat(struct ggml_context * ctx, struct ggml_tensor * a, struct ggml_tensor * b);
 void ggml_mul_mat_set_prec(struct ggml_tensor * a, enum ggml_prec prec);
+struct ggml_tensor * ggml_concat(struct ggml_context * ctx, struct ggml_tensor * a, struct ggml_tensor * b, int dim);
 struct ggml_tensor * ggml_get_rows(struct ggml_context * ctx, struct ggml_tensor * a, struct ggml_tensor * b);
 struct ggml_tensor * ggml_set_rows(struct ggml_context * ctx, struct ggml_tensor * a, struct ggml_tensor * b, struct ggml_tensor * c);
 struct ggml_tensor * ggml_silu(struct ggml_context * ctx, struct ggml_tensor * a);
@@ -104,10 +105,13 @@ struct ggml_tensor * ggml_rope_ext_inplace(struct ggml_context * ctx, struct ggm
                                    int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale, float ext_factor,
                                    float attn_factor, float beta_fast, float beta_slow);
 void ggml_rope_set_exact_freq(struct ggml_tensor * a);
+void ggml_rope_set_freq_table(struct ggml_tensor * a);  /* src[2] holds the pairs' frequencies themselves; cos / sin times attn_factor */
 struct ggml_tensor * ggml_flash_attn_ext(struct ggml_context * ctx, struct ggml_tensor * q, struct ggml_tensor * k, struct ggml_tensor * v,
                                          struct ggml_tensor * mask, float scale, float max_bias, float logit_softcap);
 void ggml_flash_attn_ext_set_prec(struct ggml_tensor * a, enum ggml_prec prec);
 void ggml_flash_attn_ext_add_sinks(struct ggml_tensor * a, struct ggml_tensor * sinks);
+/* score -= r1[h] ln(1 + r2[h] distance): r12 is f32 [heads, 2] (all r1, then all r2); the F32 mask holds distances (>= 0) of visible pairs, -inf for hidden ones */
+void ggml_flash_attn_ext_add_log_distance(struct ggml_tensor * a, struct ggml_tensor * r12);
 struct ggml_tensor * ggml_argmax(struct ggml_context * ctx, struct ggml_tensor * a);
 
 /* graphs */

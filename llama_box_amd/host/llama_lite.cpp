@@ -331,10 +331,16 @@ struct llm_layer {
     // models described layer by layer (llm_layer_cfg): norms behind the sublayers, the attention output gate, the experts and their router
     ggml_tensor *attn_post_norm = nullptr, *ffn_post_norm = nullptr, *attn_gate = nullptr;
     ggml_tensor *ffn_gate_inp = nullptr, *ffn_up_exps = nullptr, *ffn_down_exps = nullptr;
+    // ... a learned sink per head, the (r1, r2) of a distance penalty, the token-shift factors, biases of the feed-forward
+    ggml_tensor *attn_sink = nullptr, *attn_r12 = nullptr, *shift = nullptr, *ffn_gate_b = nullptr, *ffn_up_b = nullptr, *ffn_down_b = nullptr;
+    // ... latent attention: the down projection to (latent, rotated key part), the latent's norm, the per-head expansions (W_uk stored transposed per
+    // head, [dk, rank, head]: the query is taken into the latent space instead of the keys out of it), and the table of rotation frequencies
+    ggml_tensor *wdkv = nullptr, *dkv_norm = nullptr, *wuk_t = nullptr, *wuv = nullptr, *rope_freq = nullptr;
 };
 
 // one layer of a model whose config lists its layers one by one (sizes and constants may differ from layer to layer)
 enum llm_mlp_kind { LLM_MLP_NONE = 0, LLM_MLP_DENSE = 1, LLM_MLP_MOE = 2 };
+enum llm_mixer_kind { LLM_MIX_ATTN = 0, LLM_MIX_LATENT = 1 };
 struct llm_layer_cfg {
     int n_head = 0, n_head_kv = 0, dk = 0, dv = 0;  // query heads, key/value heads, per-head query/key size, per-head value size
     int rot_dims = 0;                               // leading dims of every head that are rotated, as neighbouring pairs
@@ -345,7 +351,33 @@ struct llm_layer_cfg {
     float v_lambda = 0.0f;                          // ... v <- (1 - lambda) v + lambda v_first
     bool out_gate = false;                          // heads are multiplied by sigmoid(W_g h) before the output projection
     int mlp = LLM_MLP_NONE, n_ff = 0, n_expert = 0, n_top = 0;
-    int mask_id = 0;                                // index into llm_model::mask_chunks
+    int mask_id = 0;                                // index into llm_model::mask_rules
+    // mechanisms a design may switch on layer by layer
+    int mixer = LLM_MIX_ATTN;
+    int window = 0, keep_first = 0;                 // window > 0: position i sees j <= i with i - j < window, and besides the first keep_first positions
+    bool v_unit = false;                            // every head's value is divided by its root mean square (no weight) before it is cached
+    bool dist_pen = false;                          // score -= r1_h ln(1 + r2_h (i - j)) (attn_r12)
+    bool sink_learned = false;                      // the sink's score is a learned number per head (attn_sink) instead of 0
+    bool gate_heads = false;                        // the output gate is ONE number per head (W_g has `heads` rows) instead of one per value entry
+    bool shift = false;                             // token shift: the mixer reads h + (h_prev - h) * shift, h_prev being the previous token's h (sequence state)
+    bool parallel = false;                          // x += mixer(norm(x)) + ff(norm(x)) with ONE norm, instead of two normed sublayers in a row
+    bool rms = false;                               // norms are x / sqrt(mean(x^2) + eps) * w instead of layer norms
+    bool ffn_gated_tanh = false;                    // W_down (gelu_tanh(W_gate h + b) * (W_up h + b)) + b instead of W_down gelu_erf(W_up h)
+    bool rot_half = false;                          // rotation pairs are (i, i + dims / 2) instead of neighbours
+    int kv_rank = 0, rot_dim = 0;                   // latent attention: size of the cached latent; the rotated part of a query head / the shared rotated key part
+    float yarn_factor = 0.0f, yarn_orig = 0.0f, yarn_fast = 32.0f, yarn_slow = 1.0f;  // yarn_factor > 0: frequencies blended with their 1 / factor (rope_freq)
+};
+// what a layer's positions may see: one attention mask per distinct rule of a model
+struct llm_mask_rule {
+    int chunk = 0, window = 0, keep_first = 0;
+    bool distance = false;  // the mask holds i - j for visible pairs instead of 0 (layers with a distance penalty)
+    bool operator==(const llm_mask_rule & o) const { return chunk == o.chunk && window == o.window && keep_first == o.keep_first && distance == o.distance; }
+};
+// one execution of a layer: a model may run a range of its layers several times in a row with the same weights; every run has its own cache and state
+struct llm_run {
+    int il = 0;          // the layer whose weights it uses
+    int pass = -1;       // >= 0: number of the pass through the repeated range
+    bool first = false;  // the first layer of a pass: the stream is re-projected together with the embedding output before it
 };
 
 struct tensor_plan {
@@ -377,8 +409,16 @@ struct llm_model {
     std::vector<int> layer_dev;  // ... and which of them holds layer il
     // per-layer description (empty for the uniform llama / qwen2 classes)
     std::vector<llm_layer_cfg> lcfg;
-    std::vector<int> mask_chunks;        // the distinct chunk sizes of the layers (0 = plain causal): one attention mask each
-    float embd_scale = 1.0f;
+    std::vector<llm_mask_rule> mask_rules;  // the distinct visibility rules of the layers ({} = plain causal): one attention mask each
+    std::vector<llm_run> runs;           // the order in which layers execute (one entry per layer unless a range repeats)
+    float embd_scale = 1.0f, logit_scale = 1.0f;
+    // a hashed bigram embedding added to the token embedding: row (prev * mul_prev + cur * mul_cur) mod buckets, row `buckets` for a sequence's first token
+    ggml_tensor * bigram = nullptr;
+    int bg_buckets = 0, bg_mul_prev = 0, bg_mul_cur = 0;
+    // layers [loop_start, loop_stop) run loop_times times in a row; before each pass x <- loop_in [x; embedding output] + loop_step[pass]
+    int loop_start = 0, loop_stop = 0, loop_times = 0;
+    ggml_tensor *loop_in = nullptr, *loop_step = nullptr;
+    bool has_shift = false;              // some layer keeps the previous token's normed input as sequence state
     ggml_tensor * attn_sinks = nullptr;  // zeros, one per query head: the sink's score
     ggml_type wtype = GGML_TYPE_F32;     // type of the matrices (and the default type of the cache)
     int max_embd_k = 0, max_embd_v = 0;  // widest K / V cache row over the layers
@@ -745,7 +785,18 @@ struct dir_tensor {               // one framework tensor and where its values c
     int64_t ne[3];
     std::vector<std::string> src; // checkpoint tensors, stacked along the last dim (one entry unless experts)
     float synth_gain;             // random weights: N(0, gain^2 / ne0); < 0: 1 + 0.1 N(0, 1) (norm weights)
+    bool head_transpose = false;  // the checkpoint tensor is [ne2 * ne0, ne1] (heads x rows, columns): kept as ne2 matrices [ne0, ne1] with the ROWS along dim 0
+    std::vector<float> values;    // not from the checkpoint: computed by the loader (f32 tensors)
+    float synth_lo = 0.0f, synth_hi = 0.0f;  // random weights: uniform in [lo, hi) when hi > lo (shift factors, penalties)
 };
+
+// the visibility rule of a layer gets a mask of its own unless another layer has the same
+static int mask_rule_id(llm_model * m, const llm_mask_rule & r) {
+    size_t k = 0;
+    while (k < m->mask_rules.size() && !(m->mask_rules[k] == r)) ++k;
+    if (k == m->mask_rules.size()) m->mask_rules.push_back(r);
+    return (int) k;
+}
 
 static bool parse_nigozen_config(const json_value & cfg, llm_model * m, std::string & err) {
     llm_hparams & hp = m->hp;
@@ -799,17 +850,195 @@ static bool parse_nigozen_config(const json_value & cfg, llm_model * m, std::str
             } else { err = "config: layer " + std::to_string(il) + ": unknown mlp kind"; return false; }
             if (c.n_ff <= 0) { err = "config: layer " + std::to_string(il) + ": ff missing"; return false; }
         }
-        size_t k = 0;
-        while (k < m->mask_chunks.size() && m->mask_chunks[k] != c.chunk) ++k;
-        if (k == m->mask_chunks.size()) m->mask_chunks.push_back(c.chunk);
-        c.mask_id = (int) k;
+        llm_mask_rule rule;
+        rule.chunk = c.chunk;
+        c.mask_id = mask_rule_id(m, rule);
         m->max_embd_k = std::max(m->max_embd_k, c.n_head_kv * c.dk);
         m->max_embd_v = std::max(m->max_embd_v, c.n_head_kv * c.dv);
     }
     // the uniform fields describe layer 0 (informational for per-layer models)
     hp.n_head = m->lcfg[0].n_head; hp.n_head_kv = m->lcfg[0].n_head_kv; hp.n_embd_head = m->lcfg[0].dk; hp.n_ff = m->lcfg[0].n_ff;
     hp.rope_freq_base = m->lcfg[0].rot_base;
+    for (int il = 0; il < hp.n_layer; ++il) m->runs.push_back({il, -1, false});
     return true;
+}
+
+// Zigipel: every layer is x += mixer(shift(h)) + ff(h) with h = rms_norm(x) (one norm, both sublayers read it; the mixer's copy is blended with the previous
+// token's h).  Mixers: grouped-query attention without rotation (unit-rms values, a logarithmic distance penalty, a sliding window that also keeps the first
+// tokens, a learned sink, one sigmoid gate per head), or latent attention (keys and values expanded from a cached normed latent, one rotated key part shared
+// by the heads, rotate-half layout with YaRN-blended frequencies, sliding window, learned sink).  Gated tanh-GELU feed-forward with biases.  A hashed bigram
+// embedding is added to the token embedding; a range of layers repeats; the output matrix is its own tensor and the logits are scaled.
+static bool parse_zigipel_config(const json_value & cfg, llm_model * m, std::string & err) {
+    llm_hparams & hp = m->hp;
+    snprintf(hp.arch, sizeof(hp.arch), "zigipel");
+    const json_value * layers = cfg.get("layers");
+    if (!layers || layers->kind != json_value::ARR || layers->arr.empty()) { err = "config: no layers"; return false; }
+    const json_value * v;
+    hp.n_embd = (v = cfg.get("width")) ? (int) v->number(0) : 0;
+    hp.n_vocab = (v = cfg.get("vocab")) ? (int) v->number(0) : 0;
+    hp.rms_eps = (v = cfg.path("norm", "eps")) ? (float) v->number(1e-5) : 1e-5f;
+    m->logit_scale = (v = cfg.get("logit_scale")) ? (float) v->number(1.0) : 1.0f;
+    hp.n_layer = (int) layers->arr.size();
+    hp.n_ctx_train = 1 << 20;
+    if (hp.n_embd <= 0 || hp.n_vocab <= 0) { err = "config: width / vocab missing"; return false; }
+    auto num = [&](const json_value * o, const char * k0, const char * k1, double d) { const json_value * x = o->path(k0, k1); return x ? x->number(d) : d; };
+    if (const json_value * bg = cfg.path("embedding", "bigram")) {
+        m->bg_buckets = (int) num(bg, "buckets", nullptr, 0);
+        m->bg_mul_prev = (int) num(bg, "mul_prev", nullptr, 0);
+        m->bg_mul_cur = (int) num(bg, "mul_cur", nullptr, 0);
+        if (m->bg_buckets <= 0) { err = "config: bigram embedding without buckets"; return false; }
+    }
+    if (const json_value * lp = cfg.get("loop")) {
+        m->loop_start = (int) num(lp, "start", nullptr, 0);
+        m->loop_stop = (int) num(lp, "stop", nullptr, 0);
+        m->loop_times = (int) num(lp, "times", nullptr, 1);
+        if (m->loop_start < 0 || m->loop_stop > hp.n_layer || m->loop_start >= m->loop_stop || m->loop_times < 1) { err = "config: inconsistent loop"; return false; }
+    }
+    m->lcfg.resize((size_t) hp.n_layer);
+    for (int il = 0; il < hp.n_layer; ++il) {
+        const json_value & L = layers->arr[(size_t) il];
+        llm_layer_cfg & c = m->lcfg[(size_t) il];
+        const std::string lname = "config: layer " + std::to_string(il);
+        const json_value * type = L.get("type");
+        const json_value * mx = L.get("mixer");
+        if (!type || type->kind != json_value::STR || !mx || mx->kind != json_value::OBJ) { err = lname + ": no mixer"; return false; }
+        c.parallel = c.rms = c.shift = c.sink_learned = true;
+        c.sink = true;
+        c.n_head = (int) num(mx, "heads", nullptr, 0);
+        c.dk = (int) num(mx, "dim", nullptr, 0);
+        c.dv = (int) num(mx, "vdim", nullptr, c.dk);
+        c.scale = (float) num(mx, "scale", nullptr, c.dk > 0 ? 1.0 / sqrt((double) c.dk) : 1.0);
+        c.window = (int) num(mx, "mask", "size", 0);
+        c.rot_dims = 0;
+        if (type->str == "attention") {
+            c.mixer = LLM_MIX_ATTN;
+            c.n_head_kv = (int) num(mx, "kv_heads", nullptr, c.n_head);
+            c.keep_first = (int) num(mx, "mask", "keep_first", 0);
+            c.v_unit = c.dist_pen = c.out_gate = c.gate_heads = true;
+            if (c.n_head <= 0 || c.n_head_kv <= 0 || c.n_head % c.n_head_kv || c.dk <= 0 || c.dv <= 0 || c.window < 0 || c.keep_first < 0) { err = lname + ": inconsistent attention sizes"; return false; }
+            m->max_embd_k = std::max(m->max_embd_k, c.n_head_kv * c.dk);
+            m->max_embd_v = std::max(m->max_embd_v, c.n_head_kv * c.dv);
+        } else if (type->str == "latent_attention") {
+            c.mixer = LLM_MIX_LATENT;
+            c.n_head_kv = 1;
+            c.kv_rank = (int) num(mx, "kv_rank", nullptr, 0);
+            c.rot_dim = (int) num(mx, "rot_dim", nullptr, 0);
+            c.rot_dims = c.rot_dim;  // the rotated vector is the rot_dim part of a head
+            c.rot_half = true;
+            c.rot_base = (float) num(mx, "rot", "base", 10000.0);
+            if (const json_value * sc = mx->path("rot", "scaling")) {
+                c.yarn_factor = (float) num(sc, "factor", nullptr, 1.0);
+                c.yarn_orig = (float) num(sc, "original", nullptr, 0.0);
+                c.yarn_fast = (float) num(sc, "fast", nullptr, 32.0);
+                c.yarn_slow = (float) num(sc, "slow", nullptr, 1.0);
+                if (c.yarn_factor <= 0.0f || c.yarn_orig <= 0.0f) { err = lname + ": inconsistent rotary scaling"; return false; }
+            }
+            if (c.n_head <= 0 || c.dk <= 0 || c.dv <= 0 || c.kv_rank <= 0 || c.rot_dim < 0 || (c.rot_dim & 1) || c.window < 0) { err = lname + ": inconsistent latent attention sizes"; return false; }
+            m->max_embd_k = std::max(m->max_embd_k, c.kv_rank + c.rot_dim);
+        } else { err = lname + ": unknown mixer type"; return false; }
+        const json_value * ml = L.path("mlp");
+        if (ml && ml->kind == json_value::OBJ) {
+            const json_value * kind = ml->get("kind");
+            if (!kind || kind->kind != json_value::STR || kind->str != "dense") { err = lname + ": unknown mlp kind"; return false; }
+            c.mlp = LLM_MLP_DENSE;
+            c.ffn_gated_tanh = true;
+            c.n_ff = (int) num(ml, "ff", nullptr, 0);
+            if (c.n_ff <= 0) { err = lname + ": ff missing"; return false; }
+        }
+        llm_mask_rule rule;
+        rule.window = c.window;
+        rule.keep_first = c.window > 0 ? c.keep_first : 0;
+        rule.distance = c.dist_pen;
+        c.mask_id = mask_rule_id(m, rule);
+    }
+    m->has_shift = true;
+    hp.n_head = m->lcfg[0].n_head; hp.n_head_kv = m->lcfg[0].n_head_kv; hp.n_embd_head = m->lcfg[0].dk; hp.n_ff = m->lcfg[0].n_ff;
+    hp.rope_freq_base = m->lcfg[0].rot_base;
+    // the order of execution: layers before the repeated range, the range `times` times, the rest
+    for (int il = 0; il < (m->loop_times > 0 ? m->loop_start : hp.n_layer); ++il) m->runs.push_back({il, -1, false});
+    if (m->loop_times > 0) {
+        for (int t = 0; t < m->loop_times; ++t)
+            for (int il = m->loop_start; il < m->loop_stop; ++il) m->runs.push_back({il, t, il == m->loop_start});
+        for (int il = m->loop_stop; il < hp.n_layer; ++il) m->runs.push_back({il, -1, false});
+    }
+    return true;
+}
+
+// frequency of every rotation pair, base^(-2 i / dims), blended with its 1 / factor over the ramp between the two correction dims (YaRN); computed in f64
+static std::vector<float> rope_frequencies(const llm_layer_cfg & c) {
+    const int dims = c.rot_dims, half = dims / 2;
+    std::vector<float> f((size_t) half);
+    double lo = 0.0, hi = 0.0;
+    if (c.yarn_factor > 0.0f) {
+        auto corr = [&](double turns) { return dims * log((double) c.yarn_orig / (2.0 * M_PI * turns)) / (2.0 * log((double) c.rot_base)); };
+        lo = std::max(floor(corr(c.yarn_fast)), 0.0);
+        hi = std::min(ceil(corr(c.yarn_slow)), (double) dims - 1.0);
+    }
+    for (int i = 0; i < half; ++i) {
+        const double fi = pow((double) c.rot_base, -2.0 * i / dims);
+        double v = fi;
+        if (c.yarn_factor > 0.0f) {
+            const double ramp = std::min(1.0, std::max(0.0, (i - lo) / std::max(hi - lo, 0.001)));
+            v = fi / c.yarn_factor * ramp + fi * (1.0 - ramp);
+        }
+        f[(size_t) i] = (float) v;
+    }
+    return f;
+}
+static float rope_magnitude(const llm_layer_cfg & c) { return c.yarn_factor > 0.0f ? (float) (0.1 * log((double) c.yarn_factor) + 1.0) : 1.0f; }
+
+static std::vector<dir_tensor> zigipel_plan(const llm_model * m) {
+    const llm_hparams & hp = m->hp;
+    const ggml_type wt = m->wtype;
+    const int64_t E = hp.n_embd;
+    std::vector<dir_tensor> plan;
+    auto add = [&](const std::string & name, ggml_type t, int64_t n0, int64_t n1, int64_t n2, std::vector<std::string> src, float gain) -> dir_tensor & {
+        dir_tensor d;
+        d.name = name; d.type = t; d.ne[0] = n0; d.ne[1] = n1; d.ne[2] = n2; d.src = std::move(src); d.synth_gain = gain;
+        plan.push_back(std::move(d));
+        return plan.back();
+    };
+    auto uniform = [&](dir_tensor & t, float lo, float hi) { t.synth_lo = lo; t.synth_hi = hi; };
+    add("token_embd.weight", wt, E, hp.n_vocab, 1, {"embed"}, sqrtf((float) E));
+    if (m->bg_buckets > 0) add("bigram_embd.weight", wt, E, m->bg_buckets + 1, 1, {"bigram"}, sqrtf((float) E));
+    if (m->loop_times > 0) {
+        add("loop_in.weight", wt, 2 * E, E, 1, {"loop.in"}, 1.4f);
+        add("loop_step.weight", GGML_TYPE_F32, E, m->loop_times, 1, {"loop.step"}, 0.3f * sqrtf((float) E));
+    }
+    for (int il = 0; il < hp.n_layer; ++il) {
+        const llm_layer_cfg & c = m->lcfg[(size_t) il];
+        const std::string p = "blk." + std::to_string(il) + ".", q = "l" + std::to_string(il) + ".";
+        const int64_t H = c.n_head;
+        add(p + "attn_norm.weight", GGML_TYPE_F32, E, 1, 1, {q + "norm1"}, -1.0f);
+        uniform(add(p + "shift.weight", GGML_TYPE_F32, E, 1, 1, {q + "shift"}, 0.0f), 0.0f, 1.0f);
+        add(p + "attn_sink.weight", GGML_TYPE_F32, H, 1, 1, {q + "mix.sink"}, sqrtf((float) H));
+        if (c.mixer == LLM_MIX_ATTN) {
+            add(p + "attn_q.weight", wt, E, H * c.dk, 1, {q + "mix.q"}, 2.0f);
+            add(p + "attn_k.weight", wt, E, (int64_t) c.n_head_kv * c.dk, 1, {q + "mix.k"}, 2.0f);
+            add(p + "attn_v.weight", wt, E, (int64_t) c.n_head_kv * c.dv, 1, {q + "mix.v"}, 1.0f);
+            add(p + "attn_gate.weight", wt, E, H, 1, {q + "mix.g"}, 1.0f);
+            uniform(add(p + "attn_dist.weight", GGML_TYPE_F32, H, 1, 2, {q + "mix.r1", q + "mix.r2"}, 0.0f), 0.1f, 1.0f);  // r1 of every head, then r2 of every head
+        } else {
+            add(p + "attn_q.weight", wt, E, H * (c.dk + c.rot_dim), 1, {q + "mix.q"}, 2.0f);
+            add(p + "attn_kv_a.weight", wt, E, c.kv_rank + c.rot_dim, 1, {q + "mix.dkv"}, 1.0f);
+            add(p + "attn_kv_a_norm.weight", GGML_TYPE_F32, c.kv_rank, 1, 1, {q + "mix.dkv.norm"}, -1.0f);
+            add(p + "attn_k_b_t.weight", wt, c.dk, c.kv_rank, H, {q + "mix.uk"}, 1.0f).head_transpose = true;
+            add(p + "attn_v_b.weight", wt, c.kv_rank, c.dv, H, {q + "mix.uv"}, 1.0f);
+            if (c.rot_dim > 0) add(p + "rope_freq.weight", GGML_TYPE_F32, c.rot_dim / 2, 1, 1, {}, 0.0f).values = rope_frequencies(c);
+        }
+        add(p + "attn_output.weight", wt, H * c.dv, E, 1, {q + "mix.o"}, 1.0f);
+        if (c.mlp == LLM_MLP_DENSE) {
+            add(p + "ffn_gate.weight", wt, E, c.n_ff, 1, {q + "mlp.gate"}, 1.0f);
+            add(p + "ffn_gate.bias", GGML_TYPE_F32, c.n_ff, 1, 1, {q + "mlp.gate.b"}, 0.3f * sqrtf((float) c.n_ff));
+            add(p + "ffn_up.weight", wt, E, c.n_ff, 1, {q + "mlp.up"}, 1.0f);
+            add(p + "ffn_up.bias", GGML_TYPE_F32, c.n_ff, 1, 1, {q + "mlp.up.b"}, 0.3f * sqrtf((float) c.n_ff));
+            add(p + "ffn_down.weight", wt, c.n_ff, E, 1, {q + "mlp.down"}, 1.0f);
+            add(p + "ffn_down.bias", GGML_TYPE_F32, E, 1, 1, {q + "mlp.down.b"}, 0.3f * sqrtf((float) E));
+        }
+    }
+    add("output_norm.weight", GGML_TYPE_F32, E, 1, 1, {"final.norm"}, -1.0f);
+    add("output.weight", wt, E, hp.n_vocab, 1, {"head"}, 1.0f);
+    return plan;
 }
 
 static std::vector<dir_tensor> nigozen_plan(const llm_model * m) {
@@ -818,7 +1047,9 @@ static std::vector<dir_tensor> nigozen_plan(const llm_model * m) {
     const int64_t E = hp.n_embd;
     std::vector<dir_tensor> plan;
     auto add = [&](const std::string & name, ggml_type t, int64_t n0, int64_t n1, int64_t n2, std::vector<std::string> src, float gain) {
-        plan.push_back({name, t, {n0, n1, n2}, std::move(src), gain});
+        dir_tensor d;
+        d.name = name; d.type = t; d.ne[0] = n0; d.ne[1] = n1; d.ne[2] = n2; d.src = std::move(src); d.synth_gain = gain;
+        plan.push_back(std::move(d));
     };
     add("token_embd.weight", wt, E, hp.n_vocab, 1, {"embed"}, sqrtf((float) E));
     int max_head = 1;
@@ -884,22 +1115,27 @@ static llm_model * model_from_config(const json_value & cfg, const st_file * fil
     m->wtype = (ggml_type) wtype;
     std::string err;
     // the registry of model classes that are described by a config.json
+    std::vector<dir_tensor> plan;
     if (arch->str == "Nigozen") {
         if (!parse_nigozen_config(cfg, m, err)) { fprintf(stderr, "llm_model_load_dir: %s\n", err.c_str()); delete m; return nullptr; }
+        plan = nigozen_plan(m);
+    } else if (arch->str == "Zigipel") {
+        if (!parse_zigipel_config(cfg, m, err)) { fprintf(stderr, "llm_model_load_dir: %s\n", err.c_str()); delete m; return nullptr; }
+        plan = zigipel_plan(m);
     } else {
         fprintf(stderr, "llm_model_load_dir: unknown architecture \"%s\"\n", arch->str.c_str());
         delete m;
         return nullptr;
     }
-    std::vector<dir_tensor> plan = nigozen_plan(m);
     m->ctx = ggml_init({0, nullptr, true});
     for (auto & t : plan) {
         // shapes are checked against the file before anything is allocated
         if (file)
             for (auto & sname : t.src) {
                 const st_tensor * st = file->find(sname);
-                const int64_t want = t.ne[0] * t.ne[1];
-                if (!st || st->numel() != want || (st->shape.size() == 2 && (st->shape[1] != t.ne[0] || st->shape[0] != t.ne[1]))) {
+                const int64_t n_src = (int64_t) t.src.size(), want = t.ne[0] * t.ne[1] * t.ne[2] / n_src;
+                const int64_t cols = t.head_transpose ? t.ne[1] : t.ne[0], rows = t.head_transpose ? t.ne[0] * t.ne[2] : t.ne[1] * t.ne[2] / n_src;
+                if (!st || st->numel() != want || (st->shape.size() == 2 && (st->shape[1] != cols || st->shape[0] != rows))) {
                     fprintf(stderr, "llm_model_load_dir: tensor %s is missing or has another shape than the config implies\n", sname.c_str());
                     llm_model_free(m);
                     return nullptr;
@@ -916,10 +1152,13 @@ static llm_model * model_from_config(const json_value & cfg, const st_file * fil
     int tid = 0;
     for (auto & t : plan) {
         ggml_tensor * x = ggml_get_tensor(m->ctx, t.name.c_str());
-        const size_t esz = ggml_type_size(t.type), slice = (size_t) (t.ne[0] * t.ne[1]) * esz;
-        stage.assign(slice * (size_t) t.ne[2], 0);
+        const size_t esz = ggml_type_size(t.type), total = (size_t) (t.ne[0] * t.ne[1] * t.ne[2]) * esz, slice = t.src.empty() ? total : total / t.src.size();
+        stage.assign(total, 0);
         ++tid;
-        if (t.src.empty()) {
+        if (!t.values.empty()) {
+            LLM_ASSERT(t.type == GGML_TYPE_F32 && t.values.size() * 4 == total);
+            memcpy(stage.data(), t.values.data(), total);
+        } else if (t.src.empty()) {
             // zeros (the sinks)
         } else if (file) {
             for (size_t k = 0; k < t.src.size(); ++k)
@@ -928,6 +1167,23 @@ static llm_model * model_from_config(const json_value & cfg, const st_file * fil
                     llm_model_free(m);
                     return nullptr;
                 }
+            if (t.head_transpose) {  // file: [head][row r][col c]  ->  kept: [head][col c][row r] (rows along dim 0)
+                std::vector<uint8_t> tr(total);
+                const int64_t R = t.ne[0], Cc = t.ne[1];
+                for (int64_t h = 0; h < t.ne[2]; ++h)
+                    for (int64_t r = 0; r < R; ++r)
+                        for (int64_t cc = 0; cc < Cc; ++cc)
+                            memcpy(tr.data() + (size_t) ((h * Cc + cc) * R + r) * esz, stage.data() + (size_t) ((h * R + r) * Cc + cc) * esz, esz);
+                stage.swap(tr);
+            }
+        } else if (t.synth_hi > t.synth_lo) {
+            uint64_t s = seed ^ ((uint64_t) tid * 0xD1B54A32D192ED03ull);
+            const int64_t n = t.ne[0] * t.ne[1] * t.ne[2];
+            for (int64_t i = 0; i < n; ++i) {
+                const float f = bf16_to_f32(f32_to_bf16(t.synth_lo + (t.synth_hi - t.synth_lo) * u01(splitmix64(s))));
+                LLM_ASSERT(t.type == GGML_TYPE_F32);
+                memcpy(stage.data() + i * 4, &f, 4);
+            }
         } else {
             uint64_t s = seed ^ ((uint64_t) tid * 0xD1B54A32D192ED03ull);
             const int64_t n = t.ne[0] * t.ne[1] * t.ne[2];
@@ -943,11 +1199,19 @@ static llm_model * model_from_config(const json_value & cfg, const st_file * fil
     }
     // bind
     m->tok_embd = ggml_get_tensor(m->ctx, "token_embd.weight");
-    m->output = m->tok_embd;  // the output matrix is the embedding table itself
+    m->output = ggml_get_tensor(m->ctx, "output.weight");
+    if (!m->output) m->output = m->tok_embd;  // no output matrix of its own: the embedding table itself
     m->output_norm = ggml_get_tensor(m->ctx, "output_norm.weight");
     m->attn_sinks = ggml_get_tensor(m->ctx, "attn_sinks.weight");
+    m->bigram = ggml_get_tensor(m->ctx, "bigram_embd.weight");
+    m->loop_in = ggml_get_tensor(m->ctx, "loop_in.weight");
+    m->loop_step = ggml_get_tensor(m->ctx, "loop_step.weight");
     m->layers.resize((size_t) m->hp.n_layer);
     uint64_t sbytes = ggml_nbytes(m->tok_embd) + ggml_nbytes(m->output_norm);
+    if (m->output != m->tok_embd) sbytes = ggml_nbytes(m->output) + ggml_nbytes(m->output_norm) + ggml_row_size(m->tok_embd->type, m->hp.n_embd) * (m->bigram ? 2 : 1);
+    std::vector<int> times_run((size_t) m->hp.n_layer, 0);
+    for (const llm_run & r : m->runs) times_run[(size_t) r.il]++;
+    if (m->loop_in) sbytes += (uint64_t) m->loop_times * (ggml_nbytes(m->loop_in) + ggml_row_size(GGML_TYPE_F32, m->hp.n_embd));
     for (int il = 0; il < m->hp.n_layer; ++il) {
         const std::string p = "blk." + std::to_string(il) + ".";
         auto g = [&](const char * s) { return ggml_get_tensor(m->ctx, (p + s).c_str()); };
@@ -957,8 +1221,12 @@ static llm_model * model_from_config(const json_value & cfg, const st_file * fil
         L.wv = g("attn_v.weight"); L.attn_gate = g("attn_gate.weight"); L.wo = g("attn_output.weight");
         L.ffn_norm = g("ffn_norm.weight"); L.ffn_post_norm = g("ffn_post_norm.weight"); L.ffn_up = g("ffn_up.weight"); L.ffn_down = g("ffn_down.weight");
         L.ffn_gate_inp = g("ffn_gate_inp.weight"); L.ffn_up_exps = g("ffn_up_exps.weight"); L.ffn_down_exps = g("ffn_down_exps.weight");
-        for (ggml_tensor * t : {L.attn_norm, L.attn_post_norm, L.wq, L.wk, L.wv, L.attn_gate, L.wo, L.ffn_norm, L.ffn_post_norm, L.ffn_up, L.ffn_down, L.ffn_gate_inp})
-            if (t) sbytes += ggml_nbytes(t);
+        L.attn_sink = g("attn_sink.weight"); L.attn_r12 = g("attn_dist.weight"); L.shift = g("shift.weight");
+        L.ffn_gate = g("ffn_gate.weight"); L.ffn_gate_b = g("ffn_gate.bias"); L.ffn_up_b = g("ffn_up.bias"); L.ffn_down_b = g("ffn_down.bias");
+        L.wdkv = g("attn_kv_a.weight"); L.dkv_norm = g("attn_kv_a_norm.weight"); L.wuk_t = g("attn_k_b_t.weight"); L.wuv = g("attn_v_b.weight"); L.rope_freq = g("rope_freq.weight");
+        for (ggml_tensor * t : {L.attn_norm, L.attn_post_norm, L.wq, L.wk, L.wv, L.attn_gate, L.wo, L.ffn_norm, L.ffn_post_norm, L.ffn_up, L.ffn_down, L.ffn_gate_inp,
+                                L.attn_sink, L.attn_r12, L.shift, L.ffn_gate, L.ffn_gate_b, L.ffn_up_b, L.ffn_down_b, L.wdkv, L.dkv_norm, L.wuk_t, L.wuv, L.rope_freq})
+            if (t) sbytes += ggml_nbytes(t) * (uint64_t) std::max(1, times_run[(size_t) il]);  // (a layer of a repeated range is streamed once per run)
         if (c.mlp == LLM_MLP_MOE) sbytes += (ggml_nbytes(L.ffn_up_exps) + ggml_nbytes(L.ffn_down_exps)) / (uint64_t) c.n_expert * (uint64_t) c.n_top;
         if (c.v_mix) {  // the blend factor is a scalar of the checkpoint, read once
             float lam = 0.5f;
@@ -1041,6 +1309,17 @@ static void mask_row_chunked(float * __restrict__ row, const int n_kv, const int
         row[j] = v ? vis : hid;
     }
 }
+// a sliding window that also keeps the first positions: cell j is visible to position p when pos_j <= p and (p - pos_j < window or pos_j < keep_first).
+// A visible cell's entry is 0, or — `distance` — p - pos_j itself, for layers whose scores carry a penalty on the distance
+static void mask_row_window(float * __restrict__ row, const int n_kv, const int32_t * __restrict__ cpos, const int32_t * __restrict__ cseq, const int32_t s, const int32_t p,
+                            const int32_t window, const int32_t keep_first, const bool distance, const float hid) {
+    const uint32_t pu = (uint32_t) p, wu = window > 0 ? (uint32_t) window : 0xFFFFFFFFu, ku = (uint32_t) keep_first;
+    for (int j = 0; j < n_kv; ++j) {
+        const uint32_t d = (uint32_t) (p - cpos[j]);  // (an empty cell's -1 gives p + 1: hidden by the first test)
+        const bool v = (cseq[j] == s) & ((uint32_t) cpos[j] <= pu) & ((d < wu) | ((uint32_t) cpos[j] < ku));
+        row[j] = v ? (distance ? (float) d : 0.0f) : hid;
+    }
+}
 #pragma GCC pop_options
 
 struct kv_cell {
@@ -1054,11 +1333,14 @@ struct seg_io {
     ggml_tensor *tokens = nullptr, *pos = nullptr, *mask = nullptr, *k_idxs = nullptr, *v_idxs = nullptr, *out_ids = nullptr, *resid = nullptr;
     ggml_tensor * out = nullptr;  // l_out of the segment's last layer, or the logits
     std::vector<ggml_tensor *> masks;  // models whose layers differ in what they may see: one mask per distinct rule (masks[0] == mask)
+    ggml_tensor * bigram_rows = nullptr;  // row of the bigram table per token (hashed on the host from the previous and the current token)
+    // token shift: per token the row of [h of this batch | state rows] that holds the previous token's h; per sequence of the batch its last token and its state row
+    ggml_tensor *shift_src = nullptr, *shift_last = nullptr, *shift_slot = nullptr;
 };
 
 struct graph_key {
-    int n_tokens = -1, n_kv = -1, n_outputs = -1;
-    bool operator==(const graph_key & o) const { return n_tokens == o.n_tokens && n_kv == o.n_kv && n_outputs == o.n_outputs; }
+    int n_tokens = -1, n_kv = -1, n_outputs = -1, n_seqs = -1;  // n_seqs: distinct sequences of the batch (models with sequence state; else 0)
+    bool operator==(const graph_key & o) const { return n_tokens == o.n_tokens && n_kv == o.n_kv && n_outputs == o.n_outputs && n_seqs == o.n_seqs; }
 };
 
 struct llm_context {
@@ -1070,8 +1352,13 @@ struct llm_context {
     // KV cache
     ggml_context * ctx_kv = nullptr;
     ggml_backend_buffer_t buf_kv = nullptr;
-    std::vector<ggml_tensor *> k_l, v_l;
+    std::vector<ggml_tensor *> k_l, v_l;  // one pair per layer RUN (a repeated layer has a cache per pass); v is null where the values are a part of the K rows
     std::vector<kv_cell> cells;
+    // sequence state of models that have it: the previous token's normed layer input per (run, sequence) — [n_embd, n_seq_max + 1, runs], the last row of a run
+    // stays zero (what a sequence's first token reads) — and the previous token id per sequence (the bigram embedding's hash)
+    ggml_tensor * shift_state = nullptr;
+    std::vector<int32_t> seq_prev_tok;
+    int n_seq_max = 0;
     std::vector<int32_t> mask_cpos, mask_cseq;  // the cells' fields as arrays (mask rows are filled from them)
     int kv_head = 0;
     int used_max = 0;           // one past the highest occupied cell; < 0: unknown (cells were freed), recounted by the next batch
@@ -1081,6 +1368,7 @@ struct llm_context {
     ggml_cgraph * gf = nullptr;
     graph_key key;
     ggml_tensor *inp_tokens = nullptr, *inp_pos = nullptr, *inp_mask = nullptr, *inp_k_idxs = nullptr, *inp_v_idxs = nullptr, *inp_out_ids = nullptr;
+    ggml_tensor *inp_bigram = nullptr, *inp_shift_src = nullptr, *inp_shift_last = nullptr, *inp_shift_slot = nullptr;
     std::vector<ggml_tensor *> inp_masks;  // all masks of the graph (inp_masks[0] == inp_mask)
     ggml_tensor * t_logits = nullptr;
     // outputs
@@ -1131,7 +1419,7 @@ static ggml_tensor * named(ggml_tensor * t, const char * base, int il) {
 }
 
 // creates the input tensors of layers [l0, l1) (+ the output head if `head`) in `ctx`
-static void make_inputs(llm_context * c, ggml_context * ctx, int l0, int l1, bool head, int n_tokens, int n_kv, int n_outputs, seg_io & io) {
+static void make_inputs(llm_context * c, ggml_context * ctx, int l0, int l1, bool head, int n_tokens, int n_kv, int n_outputs, seg_io & io, int n_seqs = 0) {
     llm_model * m = c->model;
     const llm_hparams & hp = m->hp;
     const bool fa = c->p.flash_attn != 0;
@@ -1157,9 +1445,21 @@ static void make_inputs(llm_context * c, ggml_context * ctx, int l0, int l1, boo
     io.mask = ggml_new_tensor_2d(ctx, GGML_TYPE_F32, n_kv, n_tok_pad);
     ggml_set_input(named(io.mask, "KQ_mask", -1));
     io.masks.assign(1, io.mask);
-    for (size_t k = 1; k < m->mask_chunks.size(); ++k) {
+    for (size_t k = 1; k < m->mask_rules.size(); ++k) {
         io.masks.push_back(ggml_new_tensor_2d(ctx, GGML_TYPE_F32, n_kv, n_tok_pad));
         ggml_set_input(named(io.masks.back(), "KQ_mask_chunked", (int) k));
+    }
+    if (m->bigram) {
+        io.bigram_rows = ggml_new_tensor_1d(ctx, GGML_TYPE_I32, n_tokens);
+        ggml_set_input(named(io.bigram_rows, "inp_bigram_rows", -1));
+    }
+    if (m->has_shift) {
+        io.shift_src = ggml_new_tensor_1d(ctx, GGML_TYPE_I32, n_tokens);
+        ggml_set_input(named(io.shift_src, "shift_src", -1));
+        io.shift_last = ggml_new_tensor_1d(ctx, GGML_TYPE_I32, std::max(1, n_seqs));
+        ggml_set_input(named(io.shift_last, "shift_last_rows", -1));
+        io.shift_slot = ggml_new_tensor_1d(ctx, GGML_TYPE_I64, std::max(1, n_seqs));
+        ggml_set_input(named(io.shift_slot, "shift_slots", -1));
     }
     io.k_idxs = ggml_new_tensor_1d(ctx, GGML_TYPE_I64, n_tokens);
     ggml_set_input(named(io.k_idxs, "k_idxs", -1));
@@ -1290,88 +1590,203 @@ static ggml_tensor * build_moe(ggml_context * ctx, ggml_cgraph * gf, const llm_l
     return named(out, "ffn_moe_out", il);
 }
 
+// the norm of a per-layer model: x / sqrt(mean(x^2) + eps) * w, or the layer norm (x - mean) / sqrt(var + eps) * w
+static ggml_tensor * norm_w(ggml_context * ctx, const llm_layer_cfg & lc, ggml_tensor * x, ggml_tensor * w, float eps, const char * name, int il) {
+    if (!lc.rms) return layer_norm_w(ctx, x, w, eps, name, il);
+    return named(ggml_mul(ctx, named(ggml_rms_norm(ctx, x, eps), "rnorm", il), w), name, il);
+}
+
+// token shift: what the mixer reads is h + (h_prev - h) * shift, h_prev being the previous token's h — the row before it in this batch when the
+// batch holds it, else the sequence's state row (a row of zeros for a sequence's first token): io.shift_src indexes [h rows | state rows].
+// Afterwards every sequence's last h of the batch becomes its state row.
+static ggml_tensor * build_token_shift(llm_context * c, ggml_context * ctx, ggml_cgraph * gf, ggml_tensor * h, ggml_tensor * w, int run, seg_io & io) {
+    ggml_tensor * state = ggml_view_2d(ctx, c->shift_state, h->ne[0], c->shift_state->ne[1], c->shift_state->nb[1], (size_t) run * c->shift_state->nb[2]);
+    ggml_tensor * both = named(ggml_concat(ctx, h, state, 1), "shift_rows", run);
+    ggml_tensor * prev = named(ggml_get_rows(ctx, both, io.shift_src), "shift_prev", run);
+    ggml_tensor * d = named(ggml_mul(ctx, named(ggml_sub(ctx, prev, h), "shift_diff", run), w), "shift_scaled", run);
+    ggml_tensor * out = named(ggml_add(ctx, h, d), "shift_out", run);
+    ggml_build_forward_expand(gf, out);  // (the state is read before it is overwritten)
+    ggml_tensor * last = named(ggml_get_rows(ctx, h, io.shift_last), "shift_last", run);
+    ggml_build_forward_expand(gf, named(ggml_set_rows(ctx, state, last, io.shift_slot), "shift_store", run));
+    return out;
+}
+
+// grouped-query attention of one layer run over its cache; returns the heads' outputs [dv * H, T] (gated), before the output projection
+static ggml_tensor * build_mixer_attention(llm_context * c, ggml_context * ctx, ggml_cgraph * gf, const llm_layer & L, const llm_layer_cfg & lc, ggml_tensor * cur, int il, int run,
+                                           int n_tokens, int n_kv, seg_io & io, ggml_tensor ** v_first) {
+    llm_model * m = c->model;
+    const llm_hparams & hp = m->hp;
+    const int64_t H = lc.n_head, G = lc.n_head_kv, DK = lc.dk, DV = lc.dv;
+    (void) il;
+    ggml_tensor * Qcur = named(ggml_mul_mat(ctx, L.wq, cur), "Qcur", run);
+    ggml_tensor * Kcur = named(ggml_mul_mat(ctx, L.wk, cur), "Kcur", run);
+    ggml_tensor * Vcur = named(ggml_mul_mat(ctx, L.wv, cur), "Vcur", run);
+    ggml_tensor * gate = lc.out_gate ? named(ggml_mul_mat(ctx, L.attn_gate, cur), "attn_gate", run) : nullptr;
+    Qcur = ggml_reshape_3d(ctx, Qcur, DK, H, n_tokens);
+    Kcur = ggml_reshape_3d(ctx, Kcur, DK, G, n_tokens);
+    if (lc.rot_dims > 0) {  // neighbouring pairs (2i, 2i + 1) of the leading rot_dims entries; the rest of the head passes through
+        Qcur = named(ggml_rope_ext(ctx, Qcur, io.pos, nullptr, lc.rot_dims, lc.rot_half ? GGML_ROPE_TYPE_NEOX : 0, hp.n_ctx_train, lc.rot_base, 1.0f, 0.0f, 1.0f, 32.0f, 1.0f), "Qcur_rope", run);
+        Kcur = named(ggml_rope_ext(ctx, Kcur, io.pos, nullptr, lc.rot_dims, lc.rot_half ? GGML_ROPE_TYPE_NEOX : 0, hp.n_ctx_train, lc.rot_base, 1.0f, 0.0f, 1.0f, 32.0f, 1.0f), "Kcur_rope", run);
+        ggml_rope_set_exact_freq(Qcur);  // angle = pos * base^(-2 i / dims) with the frequency itself rounded once (not ggml's running product)
+        ggml_rope_set_exact_freq(Kcur);
+    }
+    if (lc.v_unit)  // every head's value divided by its root mean square: that is what the cache keeps
+        Vcur = ggml_reshape_2d(ctx, named(ggml_rms_norm(ctx, ggml_reshape_3d(ctx, Vcur, DV, G, n_tokens), hp.rms_eps), "Vcur_unit", run), G * DV, n_tokens);
+    if (lc.v_mix) {
+        if (!*v_first) *v_first = Vcur;
+        else {
+            LLM_ASSERT((*v_first)->ne[0] == Vcur->ne[0]);
+            Vcur = named(ggml_add(ctx, named(ggml_scale(ctx, Vcur, 1.0f - lc.v_lambda), "Vcur_own", run), named(ggml_scale(ctx, *v_first, lc.v_lambda), "Vcur_first", run)), "Vcur_mixed", run);
+        }
+    }
+    ggml_build_forward_expand(gf, Qcur);
+    ggml_build_forward_expand(gf, Kcur);
+    ggml_build_forward_expand(gf, Vcur);
+    ggml_tensor * k_cache = c->k_l[(size_t) run];
+    ggml_tensor * v_cache = c->v_l[(size_t) run];
+    ggml_build_forward_expand(gf, named(ggml_set_rows(ctx, k_cache, ggml_reshape_2d(ctx, Kcur, G * DK, n_tokens), io.k_idxs), "k_store", run));
+    ggml_build_forward_expand(gf, named(ggml_set_rows(ctx, v_cache, ggml_reshape_2d(ctx, Vcur, G * DV, n_tokens), io.k_idxs), "v_store", run));  // (blended / normed values are what is kept)
+    ggml_tensor * q = ggml_permute(ctx, Qcur, 0, 2, 1, 3);
+    ggml_tensor * k = ggml_view_3d(ctx, k_cache, DK, n_kv, G, ggml_row_size(k_cache->type, G * DK), ggml_row_size(k_cache->type, DK), 0);
+    ggml_tensor * v = ggml_view_3d(ctx, v_cache, DV, n_kv, G, ggml_row_size(v_cache->type, G * DV), ggml_row_size(v_cache->type, DV), 0);
+    // the F32 masks go to FLASH_ATTN_EXT as they are (no F16 cast): that is how this graph asks the backend for attention in 32-bit arithmetic
+    cur = ggml_flash_attn_ext(ctx, q, k, v, io.masks[(size_t) lc.mask_id], lc.scale, 0.0f, 0.0f);
+    ggml_flash_attn_ext_set_prec(cur, GGML_PREC_F32);
+    if (lc.sink) ggml_flash_attn_ext_add_sinks(cur, lc.sink_learned ? L.attn_sink : ggml_view_1d(ctx, m->attn_sinks, H, 0));
+    if (lc.dist_pen) ggml_flash_attn_ext_add_log_distance(cur, ggml_reshape_2d(ctx, L.attn_r12, H, 2));
+    named(cur, "fattn", run);
+    if (gate && lc.gate_heads) {  // one number per head and token
+        ggml_tensor * sg = ggml_reshape_3d(ctx, named(ggml_unary(ctx, gate, GGML_UNARY_OP_SIGMOID), "attn_gate_sigmoid", run), 1, H, n_tokens);
+        cur = named(ggml_mul(ctx, cur, sg), "attn_gated", run);
+        gate = nullptr;
+    }
+    cur = ggml_reshape_2d(ctx, cur, DV * H, n_tokens);
+    if (gate) cur = named(ggml_mul(ctx, cur, named(ggml_unary(ctx, gate, GGML_UNARY_OP_SIGMOID), "attn_gate_sigmoid", run)), "attn_gated", run);
+    return cur;
+}
+
+// latent attention of one layer run.  The cache row of a token is [c | k_r]: the normed latent (kv_rank values) and the rotated key part shared by all
+// heads.  Keys and values are never expanded: with k_h = W_uk,h c the score q_h . k_h equals (W_uk,h^T q_h) . c, so the query is taken into the latent
+// space (one small mat-mul per head), every head attends over the SAME rows [c | k_r] with the query [W_uk,h^T q_h | rot(q_r,h)], the weighted sum of
+// the latents comes back, and W_uv,h expands it to the head's value.  Returns [dv * H, T].
+static ggml_tensor * build_mixer_latent(llm_context * c, ggml_context * ctx, ggml_cgraph * gf, const llm_layer & L, const llm_layer_cfg & lc, ggml_tensor * cur, int il, int run,
+                                        int n_tokens, int n_kv, seg_io & io) {
+    llm_model * m = c->model;
+    const llm_hparams & hp = m->hp;
+    const int64_t H = lc.n_head, DK = lc.dk, DR = lc.rot_dim, DV = lc.dv, R = lc.kv_rank, DQ = DK + DR, ROW = R + DR;
+    const float mag = rope_magnitude(lc);
+    (void) il;
+    ggml_tensor * Qcur = named(ggml_mul_mat(ctx, L.wq, cur), "Qcur", run);        // [DQ * H, T]: head by head [dk unrotated | dr rotated]
+    ggml_tensor * ckr = named(ggml_mul_mat(ctx, L.wdkv, cur), "kv_a", run);       // [R + DR, T]
+    ggml_tensor * lat = ggml_view_2d(ctx, ckr, R, n_tokens, ckr->nb[1], 0);
+    lat = named(ggml_mul(ctx, named(ggml_rms_norm(ctx, lat, hp.rms_eps), "kv_a_rnorm", run), L.dkv_norm), "kv_latent", run);
+    ggml_tensor * krow = lat;
+    ggml_tensor * q_rot = nullptr;
+    if (DR > 0) {
+        ggml_tensor * kr = ggml_view_3d(ctx, ckr, DR, 1, n_tokens, ckr->nb[1], ckr->nb[1], (size_t) R * sizeof(float));
+        kr = named(ggml_rope_ext(ctx, kr, io.pos, L.rope_freq, (int) DR, GGML_ROPE_TYPE_NEOX, hp.n_ctx_train, lc.rot_base, 1.0f, 0.0f, mag, 32.0f, 1.0f), "k_rot", run);
+        ggml_rope_set_freq_table(kr);
+        krow = named(ggml_concat(ctx, lat, ggml_reshape_2d(ctx, kr, DR, n_tokens), 0), "kv_row", run);
+        q_rot = ggml_view_3d(ctx, Qcur, DR, H, n_tokens, (size_t) DQ * sizeof(float), Qcur->nb[1], (size_t) DK * sizeof(float));
+        q_rot = named(ggml_rope_ext(ctx, q_rot, io.pos, L.rope_freq, (int) DR, GGML_ROPE_TYPE_NEOX, hp.n_ctx_train, lc.rot_base, 1.0f, 0.0f, mag, 32.0f, 1.0f), "q_rot", run);
+        ggml_rope_set_freq_table(q_rot);
+    }
+    ggml_build_forward_expand(gf, krow);
+    ggml_tensor * k_cache = c->k_l[(size_t) run];
+    ggml_build_forward_expand(gf, named(ggml_set_rows(ctx, k_cache, krow, io.k_idxs), "kv_store", run));
+    // the unrotated part of every head's query, [dk, T, H] seen through strides, times W_uk,h^T -> [R, T, H]
+    ggml_tensor * q_nope = ggml_view_3d(ctx, Qcur, DK, n_tokens, H, Qcur->nb[1], (size_t) DQ * sizeof(float), 0);
+    ggml_tensor * q_lat = named(ggml_mul_mat(ctx, L.wuk_t, q_nope), "q_latent", run);
+    ggml_tensor * q = ggml_permute(ctx, q_lat, 0, 2, 1, 3);  // [R, H, T]
+    if (q_rot) q = named(ggml_concat(ctx, q, q_rot, 0), "q_row", run);  // [R + DR, H, T]
+    else q = named(ggml_cont(ctx, q), "q_row", run);
+    ggml_tensor * k = ggml_view_3d(ctx, k_cache, ROW, n_kv, 1, ggml_row_size(k_cache->type, ROW), ggml_row_size(k_cache->type, ROW), 0);
+    ggml_tensor * v = ggml_view_3d(ctx, k_cache, R, n_kv, 1, ggml_row_size(k_cache->type, ROW), ggml_row_size(k_cache->type, ROW), 0);  // the latent part of the same rows
+    ggml_tensor * att = ggml_flash_attn_ext(ctx, ggml_permute(ctx, q, 0, 2, 1, 3), k, v, io.masks[(size_t) lc.mask_id], lc.scale, 0.0f, 0.0f);  // [R, H, T]
+    ggml_flash_attn_ext_set_prec(att, GGML_PREC_F32);
+    if (lc.sink) ggml_flash_attn_ext_add_sinks(att, lc.sink_learned ? L.attn_sink : ggml_view_1d(ctx, m->attn_sinks, H, 0));
+    named(att, "fattn", run);
+    ggml_tensor * o = named(ggml_mul_mat(ctx, L.wuv, ggml_permute(ctx, att, 0, 2, 1, 3)), "v_expand", run);  // [DV, T, H]
+    return named(ggml_cont_2d(ctx, ggml_permute(ctx, o, 0, 2, 1, 3), DV * H, n_tokens), "attn_heads", run);
+}
+
+static ggml_tensor * build_ffn(ggml_context * ctx, ggml_cgraph * gf, const llm_layer & L, const llm_layer_cfg & lc, ggml_tensor * cur, int il, int run) {
+    if (lc.mlp == LLM_MLP_MOE) return build_moe(ctx, gf, L, lc, cur, il);
+    if (lc.ffn_gated_tanh) {
+        ggml_tensor * g = named(ggml_add(ctx, named(ggml_mul_mat(ctx, L.ffn_gate, cur), "ffn_gate", run), L.ffn_gate_b), "ffn_gate_b", run);
+        ggml_tensor * u = named(ggml_add(ctx, named(ggml_mul_mat(ctx, L.ffn_up, cur), "ffn_up", run), L.ffn_up_b), "ffn_up_b", run);
+        cur = named(ggml_mul(ctx, named(ggml_unary(ctx, g, GGML_UNARY_OP_GELU), "ffn_gelu", run), u), "ffn_act", run);
+        return named(ggml_add(ctx, named(ggml_mul_mat(ctx, L.ffn_down, cur), "ffn_down", run), L.ffn_down_b), "ffn_out", run);
+    }
+    cur = named(ggml_mul_mat(ctx, L.ffn_up, cur), "ffn_up", run);
+    cur = named(ggml_unary(ctx, cur, GGML_UNARY_OP_GELU_ERF), "ffn_gelu", run);
+    return named(ggml_mul_mat(ctx, L.ffn_down, cur), "ffn_out", run);
+}
+
 static void build_layerwise(llm_context * c, ggml_context * ctx, ggml_cgraph * gf, int n_tokens, int n_kv, seg_io & io) {
     llm_model * m = c->model;
     const llm_hparams & hp = m->hp;
     const float eps = hp.rms_eps;
-    // the F32 masks go to FLASH_ATTN_EXT as they are (no F16 cast): that is how this graph asks the backend for attention in 32-bit arithmetic
-    const std::vector<ggml_tensor *> & mask_cnv = io.masks;
     ggml_tensor * inpL = named(ggml_get_rows(ctx, m->tok_embd, io.tokens), "inp_embd", -1);
     if (m->embd_scale != 1.0f) inpL = named(ggml_scale(ctx, inpL, m->embd_scale), "inp_scaled", -1);
+    if (m->bigram) inpL = named(ggml_add(ctx, inpL, named(ggml_get_rows(ctx, m->bigram, io.bigram_rows), "inp_bigram", -1)), "inp_sum", -1);
+    ggml_tensor * const embd_out = inpL;
     ggml_tensor * v_first = nullptr;
-    for (int il = 0; il < hp.n_layer; ++il) {
+    const int n_runs = (int) m->runs.size();
+    for (int run = 0; run < n_runs; ++run) {
+        const int il = m->runs[(size_t) run].il;
         const llm_layer & L = m->layers[(size_t) il];
         const llm_layer_cfg & lc = m->lcfg[(size_t) il];
-        const int64_t H = lc.n_head, G = lc.n_head_kv, DK = lc.dk, DV = lc.dv;
+        const bool last = run == n_runs - 1;
+        if (m->runs[(size_t) run].first) {  // a pass through the repeated range begins: x <- W_in [x; embedding output] + step[pass]
+            inpL = named(ggml_mul_mat(ctx, m->loop_in, named(ggml_concat(ctx, inpL, embd_out, 0), "loop_cat", run)), "loop_in", run);
+            ggml_tensor * step = ggml_view_1d(ctx, m->loop_step, hp.n_embd, (size_t) m->runs[(size_t) run].pass * m->loop_step->nb[1]);
+            inpL = named(ggml_add(ctx, inpL, step), "loop_x", run);
+        }
         ggml_tensor * inpSA = inpL;
-        ggml_tensor * cur = layer_norm_w(ctx, inpL, L.attn_norm, eps, "attn_norm", il);
-        ggml_tensor * Qcur = named(ggml_mul_mat(ctx, L.wq, cur), "Qcur", il);
-        ggml_tensor * Kcur = named(ggml_mul_mat(ctx, L.wk, cur), "Kcur", il);
-        ggml_tensor * Vcur = named(ggml_mul_mat(ctx, L.wv, cur), "Vcur", il);
-        ggml_tensor * gate = lc.out_gate ? named(ggml_mul_mat(ctx, L.attn_gate, cur), "attn_gate", il) : nullptr;
-        Qcur = ggml_reshape_3d(ctx, Qcur, DK, H, n_tokens);
-        Kcur = ggml_reshape_3d(ctx, Kcur, DK, G, n_tokens);
-        if (lc.rot_dims > 0) {  // neighbouring pairs (2i, 2i + 1) of the leading rot_dims entries; the rest of the head passes through
-            Qcur = named(ggml_rope_ext(ctx, Qcur, io.pos, nullptr, lc.rot_dims, 0, hp.n_ctx_train, lc.rot_base, 1.0f, 0.0f, 1.0f, 32.0f, 1.0f), "Qcur_rope", il);
-            Kcur = named(ggml_rope_ext(ctx, Kcur, io.pos, nullptr, lc.rot_dims, 0, hp.n_ctx_train, lc.rot_base, 1.0f, 0.0f, 1.0f, 32.0f, 1.0f), "Kcur_rope", il);
-            ggml_rope_set_exact_freq(Qcur);  // angle = pos * base^(-2 i / dims) with the frequency itself rounded once (not ggml's running product)
-            ggml_rope_set_exact_freq(Kcur);
-        }
-        if (lc.v_mix) {
-            if (!v_first) v_first = Vcur;
-            else {
-                LLM_ASSERT(v_first->ne[0] == Vcur->ne[0]);
-                Vcur = named(ggml_add(ctx, named(ggml_scale(ctx, Vcur, 1.0f - lc.v_lambda), "Vcur_own", il), named(ggml_scale(ctx, v_first, lc.v_lambda), "Vcur_first", il)), "Vcur_mixed", il);
+        ggml_tensor * h = norm_w(ctx, lc, inpL, L.attn_norm, eps, "attn_norm", run);
+        ggml_tensor * cur = lc.shift ? build_token_shift(c, ctx, gf, h, L.shift, run, io) : h;
+        cur = lc.mixer == LLM_MIX_LATENT ? build_mixer_latent(c, ctx, gf, L, lc, cur, il, run, n_tokens, n_kv, io)
+                                         : build_mixer_attention(c, ctx, gf, L, lc, cur, il, run, n_tokens, n_kv, io, &v_first);
+        cur = named(ggml_mul_mat(ctx, L.wo, cur), "attn_out", run);
+        if (lc.parallel) {  // both sublayers read the one normed input (the feed-forward the unshifted one); their sum joins the stream
+            if (last && io.out_ids) {  // only the rows whose logits are wanted go on from here
+                cur = ggml_get_rows(ctx, cur, io.out_ids);
+                inpSA = ggml_get_rows(ctx, inpSA, io.out_ids);
+                h = ggml_get_rows(ctx, h, io.out_ids);
             }
+            if (lc.mlp != LLM_MLP_NONE) cur = named(ggml_add(ctx, cur, build_ffn(ctx, gf, L, lc, h, il, run)), "mix_ffn", run);
+            inpL = named(ggml_add(ctx, inpSA, cur), "l_out", run);
+            continue;
         }
-        ggml_build_forward_expand(gf, Qcur);
-        ggml_build_forward_expand(gf, Kcur);
-        ggml_build_forward_expand(gf, Vcur);
-        ggml_tensor * k_cache = c->k_l[(size_t) il];
-        ggml_tensor * v_cache = c->v_l[(size_t) il];
-        ggml_build_forward_expand(gf, named(ggml_set_rows(ctx, k_cache, ggml_reshape_2d(ctx, Kcur, G * DK, n_tokens), io.k_idxs), "k_store", il));
-        ggml_build_forward_expand(gf, named(ggml_set_rows(ctx, v_cache, ggml_reshape_2d(ctx, Vcur, G * DV, n_tokens), io.k_idxs), "v_store", il));  // the blended values are what is kept
-        ggml_tensor * q = ggml_permute(ctx, Qcur, 0, 2, 1, 3);
-        ggml_tensor * k = ggml_view_3d(ctx, k_cache, DK, n_kv, G, ggml_row_size(k_cache->type, G * DK), ggml_row_size(k_cache->type, DK), 0);
-        ggml_tensor * v = ggml_view_3d(ctx, v_cache, DV, n_kv, G, ggml_row_size(v_cache->type, G * DV), ggml_row_size(v_cache->type, DV), 0);
-        cur = ggml_flash_attn_ext(ctx, q, k, v, mask_cnv[(size_t) lc.mask_id], lc.scale, 0.0f, 0.0f);
-        ggml_flash_attn_ext_set_prec(cur, GGML_PREC_F32);
-        if (lc.sink) ggml_flash_attn_ext_add_sinks(cur, ggml_view_1d(ctx, m->attn_sinks, H, 0));
-        named(cur, "fattn", il);
-        cur = ggml_reshape_2d(ctx, cur, DV * H, n_tokens);
-        if (gate) cur = named(ggml_mul(ctx, cur, named(ggml_unary(ctx, gate, GGML_UNARY_OP_SIGMOID), "attn_gate_sigmoid", il)), "attn_gated", il);
-        cur = named(ggml_mul_mat(ctx, L.wo, cur), "attn_out", il);
-        if (il == hp.n_layer - 1 && io.out_ids) {  // only the rows whose logits are wanted go on from here
+        if (last && io.out_ids) {
             cur = ggml_get_rows(ctx, cur, io.out_ids);
             inpSA = ggml_get_rows(ctx, inpSA, io.out_ids);
         }
-        cur = layer_norm_w(ctx, cur, L.attn_post_norm, eps, "attn_post_norm", il);
-        ggml_tensor * ffn_inp = named(ggml_add(ctx, cur, inpSA), lc.mlp == LLM_MLP_NONE ? "l_out" : "ffn_inp", il);
+        cur = norm_w(ctx, lc, cur, L.attn_post_norm, eps, "attn_post_norm", run);
+        ggml_tensor * ffn_inp = named(ggml_add(ctx, cur, inpSA), lc.mlp == LLM_MLP_NONE ? "l_out" : "ffn_inp", run);
         if (lc.mlp == LLM_MLP_NONE) { inpL = ffn_inp; continue; }
-        cur = layer_norm_w(ctx, ffn_inp, L.ffn_norm, eps, "ffn_norm", il);
-        if (lc.mlp == LLM_MLP_DENSE) {
-            cur = named(ggml_mul_mat(ctx, L.ffn_up, cur), "ffn_up", il);
-            cur = named(ggml_unary(ctx, cur, GGML_UNARY_OP_GELU_ERF), "ffn_gelu", il);
-            cur = named(ggml_mul_mat(ctx, L.ffn_down, cur), "ffn_out", il);
-        } else {
-            cur = build_moe(ctx, gf, L, lc, cur, il);
-        }
-        cur = layer_norm_w(ctx, cur, L.ffn_post_norm, eps, "ffn_post_norm", il);
-        inpL = named(ggml_add(ctx, cur, ffn_inp), "l_out", il);
+        cur = norm_w(ctx, lc, ffn_inp, L.ffn_norm, eps, "ffn_norm", run);
+        cur = build_ffn(ctx, gf, L, lc, cur, il, run);
+        cur = norm_w(ctx, lc, cur, L.ffn_post_norm, eps, "ffn_post_norm", run);
+        inpL = named(ggml_add(ctx, cur, ffn_inp), "l_out", run);
     }
-    ggml_tensor * cur = layer_norm_w(ctx, inpL, m->output_norm, eps, "result_norm", -1);
-    cur = named(ggml_mul_mat(ctx, m->output, cur), "result_output", -1);
+    const bool rms_out = !m->lcfg.empty() && m->lcfg[0].rms;
+    ggml_tensor * cur = rms_out ? named(ggml_mul(ctx, named(ggml_rms_norm(ctx, inpL, eps), "rnorm", -1), m->output_norm), "result_norm", -1)
+                                : layer_norm_w(ctx, inpL, m->output_norm, eps, "result_norm", -1);
+    cur = named(ggml_mul_mat(ctx, m->output, cur), m->logit_scale != 1.0f ? "result_unscaled" : "result_output", -1);
+    if (m->logit_scale != 1.0f) cur = named(ggml_scale(ctx, cur, m->logit_scale), "result_output", -1);
     ggml_set_output(cur);
     ggml_build_forward_expand(gf, cur);
     io.out = cur;
 }
 
-static void build_graph(llm_context * c, int n_tokens, int n_kv, int n_outputs) {
+static void build_graph(llm_context * c, int n_tokens, int n_kv, int n_outputs, int n_seqs = 0) {
     if (c->ctx_compute) ggml_free(c->ctx_compute);
     c->ctx_compute = ggml_init({0, nullptr, true});
     ggml_cgraph * gf = ggml_new_graph_custom(c->ctx_compute, 8192, false);
     seg_io io;
-    make_inputs(c, c->ctx_compute, 0, c->model->hp.n_layer, true, n_tokens, n_kv, n_outputs, io);
+    make_inputs(c, c->ctx_compute, 0, c->model->hp.n_layer, true, n_tokens, n_kv, n_outputs, io, n_seqs);
     if (!c->model->lcfg.empty()) build_layerwise(c, c->ctx_compute, gf, n_tokens, n_kv, io);
     else build_segment(c, c->ctx_compute, gf, 0, c->model->hp.n_layer, true, n_tokens, n_kv, io);
     c->inp_masks = io.masks;
@@ -1381,6 +1796,10 @@ static void build_graph(llm_context * c, int n_tokens, int n_kv, int n_outputs) 
     c->inp_k_idxs = io.k_idxs;
     c->inp_v_idxs = io.v_idxs;
     c->inp_out_ids = io.out_ids;
+    c->inp_bigram = io.bigram_rows;
+    c->inp_shift_src = io.shift_src;
+    c->inp_shift_last = io.shift_last;
+    c->inp_shift_slot = io.shift_slot;
     c->t_logits = io.out;
     c->gf = gf;
 }
@@ -1425,18 +1844,26 @@ extern "C" struct llm_context * llm_context_new(struct llm_model * m, ggml_backe
         return nullptr;
     }
     c->ctx_kv = ggml_init({0, nullptr, true});
-    for (int il = 0; il < hp.n_layer; ++il) {
-        // (a model described layer by layer: every layer's cache rows have that layer's own widths, K and V apart)
-        const int64_t row_k = layerwise ? (int64_t) m->lcfg[(size_t) il].n_head_kv * m->lcfg[(size_t) il].dk : n_embd_k;
-        const int64_t row_v = layerwise ? (int64_t) m->lcfg[(size_t) il].n_head_kv * m->lcfg[(size_t) il].dv : n_embd_k;
+    const int n_runs = layerwise ? (int) m->runs.size() : hp.n_layer;
+    for (int run = 0; run < n_runs; ++run) {
+        // (a model described layer by layer: every layer RUN has a cache of its own, its rows as wide as that layer's keys and values; a latent-attention
+        // layer keeps ONE row [latent | rotated key part] per token and no values beside it)
+        const llm_layer_cfg * lc = layerwise ? &m->lcfg[(size_t) m->runs[(size_t) run].il] : nullptr;
+        const bool latent = lc && lc->mixer == LLM_MIX_LATENT;
+        const int64_t row_k = latent ? (int64_t) lc->kv_rank + lc->rot_dim : lc ? (int64_t) lc->n_head_kv * lc->dk : n_embd_k;
+        const int64_t row_v = lc ? (int64_t) lc->n_head_kv * lc->dv : n_embd_k;
         ggml_tensor * k = ggml_new_tensor_2d(c->ctx_kv, type_k, row_k, c->p.n_ctx);
-        ggml_tensor * v = c->p.flash_attn ? ggml_new_tensor_2d(c->ctx_kv, type_v, row_v, c->p.n_ctx)
+        ggml_tensor * v = latent ? nullptr
+                        : c->p.flash_attn ? ggml_new_tensor_2d(c->ctx_kv, type_v, row_v, c->p.n_ctx)
                                           : ggml_new_tensor_2d(c->ctx_kv, GGML_TYPE_F16, c->p.n_ctx, n_embd_k);
-        named(k, "cache_k_l", il);
-        named(v, "cache_v_l", il);
+        named(k, "cache_k_l", run);
+        if (v) named(v, "cache_v_l", run);
         c->k_l.push_back(k);
         c->v_l.push_back(v);
     }
+    c->n_seq_max = c->p.n_seq_max > 0 ? c->p.n_seq_max : 8;
+    if (m->has_shift || m->bigram) c->seq_prev_tok.assign((size_t) c->n_seq_max, -1);
+    if (m->has_shift) c->shift_state = named(ggml_new_tensor_3d(c->ctx_kv, GGML_TYPE_F32, hp.n_embd, c->n_seq_max + 1, n_runs), "shift_state", -1);
     c->buf_kv = ggml_backend_alloc_ctx_tensors_from_buft(c->ctx_kv, c->buft);
     if (!c->buf_kv) {
         fprintf(stderr, "llm_context_new: failed to allocate the KV cache\n");
@@ -1448,7 +1875,7 @@ extern "C" struct llm_context * llm_context_new(struct llm_model * m, ggml_backe
     c->used_max = 0;
     c->galloc = ggml_gallocr_new(c->buft);
     // reserve the worst-case graph (full micro-batch over the full cache) so later graphs re-use one buffer
-    build_graph(c, std::min(c->p.n_ubatch, c->p.n_ctx), c->p.n_ctx, std::min(c->p.n_ubatch, c->p.n_ctx));
+    build_graph(c, std::min(c->p.n_ubatch, c->p.n_ctx), c->p.n_ctx, std::min(c->p.n_ubatch, c->p.n_ctx), m->has_shift ? std::min(c->n_seq_max, std::min(c->p.n_ubatch, c->p.n_ctx)) : 0);
     if (!ggml_gallocr_reserve(c->galloc, c->gf)) {
         fprintf(stderr, "llm_context_new: failed to reserve the compute buffer\n");
         llm_context_free(c);
@@ -1460,7 +1887,8 @@ extern "C" struct llm_context * llm_context_new(struct llm_model * m, ggml_backe
         if (hbuft) {
             const size_t nub = (size_t) std::min(c->p.n_ubatch, c->p.n_ctx);
             const size_t n_tok_pad = (nub + 63) / 64 * 64;
-            size_t in_bytes = nub * (4 + 4 + 8 + 4) + std::max<size_t>(1, m->mask_chunks.size()) * (n_tok_pad * (size_t) c->p.n_ctx * 4 + 64) + 256;
+            size_t in_bytes = nub * (4 + 4 + 8 + 4) + std::max<size_t>(1, m->mask_rules.size()) * (n_tok_pad * (size_t) c->p.n_ctx * 4 + 64) + 256;
+            in_bytes += nub * (4 + 4) + (size_t) c->n_seq_max * (4 + 8) + 4 * 64;  // bigram rows, token-shift sources, the sequences' last rows and state rows
             if (!c->p.flash_attn) in_bytes += nub * (size_t) n_embd_k * 8;
             in_bytes = (in_bytes + 255) / 256 * 256;
             c->pin_out_rows = 64;
@@ -1555,6 +1983,7 @@ static int kv_apply_shift(llm_context * c, const std::vector<int32_t> & delta) {
 // (llama.cpp defers that to the next llama_decode's memory update — same result).  Returns 0, or -2 if the shift graph failed.
 extern "C" int llm_kv_seq_add(struct llm_context * c, int seq_id, int p0, int p1, int delta) {
     if (!c->ls.empty()) return -2;  // (the K-shift graph is not cut over devices in this harness)
+    if (c->model->has_shift) return -2;  // (sequence state beside the cache: positions of such a model do not move)
     if (p0 < 0) p0 = 0;
     if (p1 < 0) p1 = INT32_MAX;
     if (delta == 0) return 0;
@@ -1782,11 +2211,40 @@ static int decode_ubatch(llm_context * c, int n_tokens, const int32_t * tokens, 
         return rc;
     }
 
-    graph_key key{n_tokens, n_kv, n_out_graph};
+    // sequence state (models with a hashed bigram embedding / token shift): where every token finds its predecessor — the row before it in this
+    // micro-batch, or its sequence's state — and which token of each sequence is the last one here.  A token at position 0 has no predecessor
+    std::vector<int32_t> bigram_rows, shift_src, shift_last;
+    std::vector<int64_t> shift_slot;
+    std::vector<int32_t> new_prev_tok;
+    if (m->has_shift || m->bigram) {
+        const int S = c->n_seq_max;
+        std::vector<int> last_in_batch((size_t) S, -1);
+        new_prev_tok = c->seq_prev_tok;
+        bigram_rows.resize((size_t) n_tokens);
+        shift_src.resize((size_t) n_tokens);
+        for (int i = 0; i < n_tokens; ++i) {
+            const int sq = seq_id ? seq_id[i] : 0;
+            const int before = last_in_batch[(size_t) sq];
+            const bool first = pos[i] == 0;
+            const int32_t prev_tok = before >= 0 ? tokens[before] : new_prev_tok[(size_t) sq];
+            if (first || prev_tok < 0) bigram_rows[(size_t) i] = m->bg_buckets;
+            else bigram_rows[(size_t) i] = (int32_t) (((int64_t) prev_tok * m->bg_mul_prev + (int64_t) tokens[i] * m->bg_mul_cur) % m->bg_buckets);
+            shift_src[(size_t) i] = first ? n_tokens + S : before >= 0 ? before : n_tokens + sq;  // rows of [h of the batch | state rows | zero row]
+            last_in_batch[(size_t) sq] = i;
+        }
+        for (int sq = 0; sq < S; ++sq)
+            if (last_in_batch[(size_t) sq] >= 0) {
+                shift_last.push_back(last_in_batch[(size_t) sq]);
+                shift_slot.push_back(sq);
+                new_prev_tok[(size_t) sq] = tokens[last_in_batch[(size_t) sq]];
+            }
+    }
+    const int n_seqs = m->has_shift ? (int) shift_last.size() : 0;
+    graph_key key{n_tokens, n_kv, n_out_graph, n_seqs};
     bool rebuilt = false;
     if (!(c->p.graph_reuse && key == c->key && c->gf)) {
         rebuilt = true;
-        build_graph(c, n_tokens, n_kv, n_out_graph);
+        build_graph(c, n_tokens, n_kv, n_out_graph, n_seqs);
         if (!ggml_gallocr_alloc_graph(c->galloc, c->gf)) return -2;
         c->key = key;
     }
@@ -1834,6 +2292,12 @@ static int decode_ubatch(llm_context * c, int n_tokens, const int32_t * tokens, 
         });
     }
     if (c->inp_out_ids) upload(c->inp_out_ids, (size_t) n_out_graph * 4, [&](char * d) { memcpy(d, out_ids.data(), (size_t) n_out_graph * 4); });
+    if (c->inp_bigram) upload(c->inp_bigram, (size_t) n_tokens * 4, [&](char * d) { memcpy(d, bigram_rows.data(), (size_t) n_tokens * 4); });
+    if (c->inp_shift_src) {
+        upload(c->inp_shift_src, (size_t) n_tokens * 4, [&](char * d) { memcpy(d, shift_src.data(), (size_t) n_tokens * 4); });
+        upload(c->inp_shift_last, (size_t) n_seqs * 4, [&](char * d) { memcpy(d, shift_last.data(), (size_t) n_seqs * 4); });
+        upload(c->inp_shift_slot, (size_t) n_seqs * 8, [&](char * d) { memcpy(d, shift_slot.data(), (size_t) n_seqs * 8); });
+    }
     {
         // rows beyond n_tokens are padding (GGML_KQ_MASK_PAD) that no kernel reads: they are written once when the
         // graph is (re)built and skipped on re-use, which keeps the per-step upload at n_tokens * n_kv entries
@@ -1850,12 +2314,15 @@ static int decode_ubatch(llm_context * c, int n_tokens, const int32_t * tokens, 
             cseq[j] = c->cells[j].seq;
         }
         for (size_t mk = 0; mk < c->inp_masks.size(); ++mk) {
-            const int chunk = mk < m->mask_chunks.size() ? m->mask_chunks[mk] : 0;
+            const llm_mask_rule rule = mk < m->mask_rules.size() ? m->mask_rules[mk] : llm_mask_rule();
+            const int chunk = rule.chunk;
             upload(c->inp_masks[mk], (size_t) n_kv * rows * 4, [&](char * d) {
                 float * mask = (float *) d;
                 for (size_t e = (size_t) n_kv * n_tokens; e < (size_t) n_kv * rows; ++e) mask[e] = -INFINITY;
                 for (int i = 0; i < n_tokens; ++i) {
-                    if (chunk > 0) mask_row_chunked(mask + (size_t) i * n_kv, n_kv, cpos.data(), cseq.data(), seq_id ? seq_id[i] : 0, pos[i], chunk, 0.0f, -INFINITY);
+                    if (rule.window > 0 || rule.distance)
+                        mask_row_window(mask + (size_t) i * n_kv, n_kv, cpos.data(), cseq.data(), seq_id ? seq_id[i] : 0, pos[i], rule.window, rule.keep_first, rule.distance, -INFINITY);
+                    else if (chunk > 0) mask_row_chunked(mask + (size_t) i * n_kv, n_kv, cpos.data(), cseq.data(), seq_id ? seq_id[i] : 0, pos[i], chunk, 0.0f, -INFINITY);
                     else mask_row(mask + (size_t) i * n_kv, n_kv, cpos.data(), cseq.data(), seq_id ? seq_id[i] : 0, pos[i], 0.0f, -INFINITY);
                 }
             });
@@ -1891,6 +2358,7 @@ static int decode_ubatch(llm_context * c, int n_tokens, const int32_t * tokens, 
         else if (!async_out) ggml_backend_tensor_get(c->t_logits, logits_out, 0, logit_bytes);
         *n_out_acc += n_outputs;
     }
+    if (!new_prev_tok.empty()) c->seq_prev_tok.swap(new_prev_tok);
     const double t4 = now_us();
     c->timings[0] += t1 - t0;
     c->timings[1] += t2 - t1;
@@ -1903,6 +2371,9 @@ extern "C" int llm_decode(struct llm_context * c, int n_tokens, const int32_t * 
     if (n_tokens <= 0 || !tokens || !pos) return -1;
     for (int i = 0; i < n_tokens; ++i)
         if (tokens[i] < 0 || tokens[i] >= c->model->hp.n_vocab || pos[i] < 0) return -1;
+    if (!c->seq_prev_tok.empty())  // a model with state per sequence: the ids index its state rows
+        for (int i = 0; i < n_tokens; ++i)
+            if (seq_id && (seq_id[i] < 0 || seq_id[i] >= c->n_seq_max)) return -1;
     int n_total_out = 0;
     for (int i = 0; i < n_tokens; ++i) n_total_out += (!want_logits || want_logits[i]) ? 1 : 0;
     // outputs land in the pinned area when they all fit (one sampled row per sequence: always, up to 64 sequences)

@@ -33,7 +33,7 @@ class TraceSession:
         self.n_vocab = self.H.llm_model_hparams(self.model).contents.n_vocab
         # every live request may hold a last, partly filled group of 64 cells beyond what it asked for
         n_ctx = int(max_tokens) + 64 * N_SLOTS
-        cp = L.ContextParams(n_ctx, n_ubatch, 1, 0, 1, 0, 0)
+        cp = L.ContextParams(n_ctx, n_ubatch, 1, 0, 1, 0, 0, N_SLOTS)
         self.ctx = self.H.llm_context_new(self.model, self.backend.backend, L.COMPUTE_FN(), C.byref(cp))
         if not self.ctx:
             raise RuntimeError("context creation failed")
