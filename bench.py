@@ -139,15 +139,40 @@ NIGOZEN_SIZES = {
 }
 
 
-def nigozen_config(z):
-    """layers alternate a dense and a mixture-of-experts feed-forward; every layer mixes values and is confined to chunks"""
+def nigozen_config(z, dense_only=False):
+    """layers alternate a dense and a mixture-of-experts feed-forward (dense_only: every layer dense); every layer mixes values and is confined to chunks"""
     layers = []
     for il in range(z["layers"]):
         mixer = {"heads": z["heads"], "kv_heads": z["kv"], "dim": z["hd"], "vdim": z["hd"], "mask": {"size": z["chunk"]}, "rot": {"base": 1e6, "dims": z["rot"]},
                  "scale": z["hd"] ** -0.5, "v_mix": True}
-        mlp = {"kind": "dense", "ff": z["ff"]} if il % 2 == 0 else {"kind": "moe", "expert": {"ff": z["eff"]}, "router": {"experts": z["experts"], "top": z["top"]}}
+        mlp = {"kind": "dense", "ff": z["ff"]} if (il % 2 == 0 or dense_only) else {"kind": "moe", "expert": {"ff": z["eff"]}, "router": {"experts": z["experts"], "top": z["top"]}}
         layers.append({"type": "attention", "mixer": mixer, "mlp": mlp})
     return {"architecture": "Nigozen", "embedding": {"scale": 1.0}, "layers": layers, "norm": {"eps": 1e-5}, "vocab": z["vocab"], "width": z["width"]}
+
+
+# ------------------------------------------------------------------------------------------------ --zigipel: the class with latent attention, token shift and a repeated range, beside Nigozen
+ZIGIPEL_SIZES = {
+    # width, heads, kv heads, head size, latent size, rotated part, window, kept first tokens, ff (gated: three matrices), vocab.  Four layers (latent, attention, latent, attention),
+    # the middle two run twice: six layer runs, as many as the Nigozen model beside it has layers.  s and m keep the latent row (latent + rotated part) within 128 values,
+    # l has a row of 576 values
+    "s": dict(width=1024, heads=8, kv=2, hd=64, rank=96, rot=32, window=512, keep=4, ff=2752, vocab=32000),
+    "m": dict(width=2048, heads=16, kv=4, hd=128, rank=96, rot=32, window=1024, keep=4, ff=5504, vocab=32000),
+    "l": dict(width=4096, heads=32, kv=8, hd=128, rank=512, rot=64, window=2048, keep=4, ff=9600, vocab=32000),
+}
+
+
+def zigipel_config(z):
+    def latent():
+        return {"type": "latent_attention", "mlp": {"kind": "dense", "ff": z["ff"]},
+                "mixer": {"heads": z["heads"], "dim": z["hd"], "rot_dim": z["rot"], "vdim": z["hd"], "kv_rank": z["rank"], "scale": (z["hd"] + z["rot"]) ** -0.5, "mask": {"size": z["window"]},
+                          "rot": {"base": 1e6, "dims": z["rot"], "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}}
+
+    def attention():
+        return {"type": "attention", "mlp": {"kind": "dense", "ff": z["ff"]},
+                "mixer": {"heads": z["heads"], "kv_heads": z["kv"], "dim": z["hd"], "vdim": z["hd"], "scale": z["hd"] ** -0.5, "mask": {"size": z["window"], "keep_first": z["keep"]}}}
+
+    return {"architecture": "Zigipel", "embedding": {"bigram": {"buckets": 8191, "mul_prev": 31, "mul_cur": 7}}, "layers": [latent(), attention(), latent(), attention()],
+            "loop": {"start": 1, "stop": 3, "times": 2}, "norm": {"eps": 1e-5}, "logit_scale": 0.5, "vocab": z["vocab"], "width": z["width"]}
 
 
 def bench_nigozen(args):
@@ -165,6 +190,10 @@ def bench_nigozen(args):
 
     be = L.Backend(0)
     n_prompt, n_dec, ub = args.prefill, max(8, min(args.steps, 64)), args.ubatch
+    if args.zigipel and n_prompt == 2048:
+        # decoded positions 1984 .. 2047: a model confined to chunks of 512 / 1024 / 2048 positions then sees 449 .. 512 / 961 .. 1024 / 1985 .. 2048 cells, about as many as a
+        # sliding window of the same length does (right behind a chunk's start it would see next to nothing, and the two decode steps would not compare)
+        n_prompt = 1984
     out = {"metric": "nigozen_vs_llama_tokens_per_s", "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16 (nigozen) / f16 (llama)", "data": "synthetic", "prompt": n_prompt,
            "decode_steps": n_dec, "ubatch": ub, "sizes": {}}
 
@@ -204,6 +233,26 @@ def bench_nigozen(args):
         ctx.free()
         return res
 
+    if args.zigipel:  # Zigipel beside Nigozen (all layers dense) with as many layers as Zigipel has layer runs, equal width, heads, head size and vocabulary
+        out["metric"] = "zigipel_vs_nigozen_tokens_per_s"
+        out["dtype"] = "bf16 (both)"
+        for name in args.zigipel.split(","):
+            z = ZIGIPEL_SIZES[name]
+            mz = Model(config_json=_json.dumps(zigipel_config(z)), seed=7, buft=be.buft, wtype=L.BF16)
+            r_z = run(mz, z["vocab"])
+            r_z["weight_bytes"] = int(L.host().llm_model_total_bytes(mz.m))
+            r_z["stream_bytes_per_token"] = mz.stream_bytes()
+            mz.free()
+            zn = dict(width=z["width"], layers=6, heads=z["heads"], kv=z["kv"], hd=z["hd"], rot=z["hd"] // 2, chunk=z["window"], ff=z["ff"] * 3 // 2, vocab=z["vocab"])
+            mn = Model(config_json=_json.dumps(nigozen_config(zn, dense_only=True)), seed=7, buft=be.buft, wtype=L.BF16)
+            r_n = run(mn, z["vocab"])
+            r_n["stream_bytes_per_token"] = mn.stream_bytes()
+            mn.free()
+            out["sizes"][name] = {"config": z, "zigipel": r_z, "nigozen_dense": r_n, "prefill_ratio": round(r_z["prefill_tok_s"] / r_n["prefill_tok_s"], 3),
+                                  "decode_ratio": round(r_z["decode_tok_s"] / r_n["decode_tok_s"], 3)}
+        print(_json.dumps(out))
+        be.close()
+        return
     for name in args.nigozen.split(","):
         z = NIGOZEN_SIZES[name]
         cfg = nigozen_config(z)
@@ -227,6 +276,8 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--nigozen", default="", help="comma-separated sizes (s, m, l): time prefill and decode of Nigozen models of these sizes beside llama (f16) at equal size, "
                     "print one JSON line and exit; the default workload is not run")
+    ap.add_argument("--zigipel", default="", help="comma-separated sizes (s, m, l): time prefill and decode of Zigipel models (latent + windowed attention, token shift, a repeated range) "
+                    "beside Nigozen models of equal size, print one JSON line and exit; the default workload is not run")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=8)
@@ -255,7 +306,7 @@ def main():
     ap.add_argument("--pmc-traffic", type=int, default=1, help="1: re-run a short decode under rocprofv3 --pmc FETCH_SIZE (own pass) for roofline.traffic")
     args = ap.parse_args()
 
-    if args.nigozen:
+    if args.nigozen or args.zigipel:
         bench_nigozen(args)
         return
 

@@ -1398,7 +1398,7 @@ static bool plan_rope_store(const exec_state & st, int i, rope_store_plan & pl) 
     ggml_cgraph * g = st.g;
     const ggml_tensor * rq = g->nodes[i];
     if (rq->op != GGML_OP_ROPE) return false;
-    if (rq->op_params[3] == 1) return false;  // (exact per-pair frequencies: served by the plain rope kernels)
+    if (rq->op_params[3] != 0) return false;  // (exact per-pair frequencies / a frequency table: served by the plain rope kernels)
     const ggml_tensor * q = rq->src[0];
     if (rq->type != GGML_TYPE_F32 || !ggml_abi_is_contiguous(rq) || q->type != GGML_TYPE_F32 || q->nb[0] != 4 || rq->ne[3] != 1 || rq->ne[2] < 2) return false;
     if ((rq->op_params[2] & GGML_ROPE_TYPE_MROPE) || rq->src[1]->type != GGML_TYPE_I32 || !ggml_abi_is_contiguous(rq->src[1])) return false;
@@ -1831,6 +1831,135 @@ static int sole_cache_store_of(const exec_state & st, int i, const ggml_tensor *
     return -1;
 }
 
+// ------------------------------------------------------------------------------------------------ fused steps of models with token shift / latent attention
+// elementwise result `d` written while `x` is read: legal when they are the same block (every thread reads its own element before it writes it) or apart
+static bool elementwise_safe(const ggml_tensor * d, const ggml_tensor * x) { return d->data == x->data || !ranges_overlap(d, x); }
+static bool is_row_of(const ggml_tensor * b, const ggml_tensor * x) { return is_f32_contig(b) && b->ne[0] == x->ne[0] && ggml_abi_nelements(b) == b->ne[0]; }
+
+// CONCAT(h, state; dim 1) -> GET_ROWS(., src) -> SUB(., h) -> MUL(., w) -> ADD(h, .): the token shift in one launch.  Returns the nodes consumed (0: no match)
+static int try_fuse_token_shift(exec_state & st, int i) {
+    ggml_cgraph * g = st.g;
+    const ggml_tensor * cat = g->nodes[i];
+    if (cat->op_params[0] != 1 || i + 4 >= g->n_nodes) return 0;
+    for (int k = 1; k <= 4; ++k) if (st.done[i + k]) return 0;
+    const ggml_tensor * h = cat->src[0], * state = cat->src[1];
+    const ggml_tensor * gr = g->nodes[i + 1], * sb = g->nodes[i + 2], * ml = g->nodes[i + 3], * ad = g->nodes[i + 4];
+    if (gr->op != GGML_OP_GET_ROWS || gr->src[0] != cat || sb->op != GGML_OP_SUB || sb->src[0] != gr || sb->src[1] != h || ml->op != GGML_OP_MUL || ml->src[0] != sb ||
+        ad->op != GGML_OP_ADD || ad->src[0] != h || ad->src[1] != ml) return 0;
+    const ggml_tensor * idx = gr->src[1], * w = ml->src[1];
+    if (!is_f32_contig(h) || h->ne[2] != 1 || h->ne[3] != 1 || state->type != GGML_TYPE_F32 || state->nb[0] != 4 || state->ne[0] != h->ne[0] || state->ne[2] != 1 || state->ne[3] != 1) return 0;
+    if (idx->type != GGML_TYPE_I32 || !ggml_abi_is_contiguous(idx) || ggml_abi_nelements(idx) != h->ne[1] || !is_row_of(w, h) || !is_f32_contig(ad) || !same_shape(ad, h)) return 0;
+    if (!single_use(st, cat) || !single_use(st, gr) || !single_use(st, sb) || !single_use(st, ml)) return 0;
+    if (ranges_overlap(ad, h) || ranges_overlap(ad, state) || ranges_overlap(ad, w) || ranges_overlap(ad, idx)) return 0;
+    launch_token_shift(st.c->stream, (const float *) h->data, h->ne[0], h->ne[1], TD(state), (const int32_t *) idx->data, (const float *) w->data, (float *) ad->data);
+    st.c->st.kernel_launches++;
+    st.c->st.fused_nodes += 4;
+    return 5;
+}
+
+// ADD(mat-mul, bias) -> GELU ... [mat-mul] -> ADD(mat-mul, bias) -> MUL(gelu, .): the gated activation with both biases in one launch.  The second mat-mul, when it
+// sits between, is executed early (its result may not occupy memory that is still read).  Returns true when node i is done (the rest is marked)
+static int run_node(exec_state & st, int i);
+static bool try_fuse_geglu_bias(exec_state & st, int i) {
+    ggml_cgraph * g = st.g;
+    const ggml_tensor * n = g->nodes[i];
+    const ggml_tensor * mg = n->src[0], * bg = n->src[1];
+    if (i + 3 >= g->n_nodes || mg->op != GGML_OP_MUL_MAT || !is_f32_contig(mg) || !is_f32_contig(n) || !same_shape(n, mg) || !is_row_of(bg, n)) return false;
+    const ggml_tensor * ge = g->nodes[i + 1];
+    if (st.done[i + 1] || ge->op != GGML_OP_UNARY || ge->op_params[0] != GGML_UNARY_OP_GELU || ge->src[0] != n || !single_use(st, n) || !single_use(st, ge)) return false;
+    int j = i + 2, up_at = -1;
+    auto skip_done = [&]() { while (j < g->n_nodes && st.done[j]) ++j; };
+    skip_done();
+    if (j < g->n_nodes && g->nodes[j]->op == GGML_OP_MUL_MAT) { up_at = j; ++j; skip_done(); }
+    if (j >= g->n_nodes) return false;
+    const int au_at = j;
+    const ggml_tensor * au = g->nodes[au_at];
+    if (au->op != GGML_OP_ADD || !is_f32_contig(au)) return false;
+    const ggml_tensor * mu = au->src[0], * bu = au->src[1];
+    if (mu->op != GGML_OP_MUL_MAT || !is_f32_contig(mu) || !same_shape(mu, mg) || !is_row_of(bu, n) || mu->src[1] != mg->src[1] || !single_use(st, mu)) return false;
+    if (up_at >= 0 && g->nodes[up_at] != mu) return false;
+    if (up_at < 0) {  // the second product must have run already: a node before this one, or one executed early
+        bool ready = false;
+        for (int k = std::max(0, i - 12); k < au_at && !ready; ++k) ready = g->nodes[k] == mu && (k < i || st.done[k]);
+        if (!ready) return false;
+    }
+    ++j; skip_done();
+    if (j >= g->n_nodes) return false;
+    const int m_at = j;
+    const ggml_tensor * m = g->nodes[m_at];
+    if (m->op != GGML_OP_MUL || !((m->src[0] == ge && m->src[1] == au) || (m->src[0] == au && m->src[1] == ge)) || !single_use(st, au) || !is_f32_contig(m) || !same_shape(m, n)) return false;
+    if (!elementwise_safe(m, mg) || !elementwise_safe(m, mu) || ranges_overlap(m, bg) || ranges_overlap(m, bu)) return false;
+    if (up_at >= 0) {
+        if (is_quant(mu->src[0]->type) || ranges_overlap(mu, mg) || ranges_overlap(mu, bg) || ranges_overlap(mu, bu)) return false;
+        if (run_node(st, up_at) != 1) return false;
+        mark_done(st, up_at);
+    }
+    launch_geglu_bias(st.c->stream, (const float *) mg->data, (const float *) bg->data, (const float *) mu->data, (const float *) bu->data, (float *) m->data, n->ne[0], ggml_abi_nrows(n));
+    mark_done(st, i + 1);
+    mark_done(st, au_at);
+    mark_done(st, m_at);
+    st.c->st.kernel_launches++;
+    st.c->st.fused_nodes += 3;
+    return true;
+}
+
+// ADD(y, bias) -> ADD(a, .) -> ADD(x, .): a projection's bias, the sum of two parallel sublayers and the residual in one launch.  Returns the nodes consumed
+static int try_fuse_add_chain(exec_state & st, int i) {
+    ggml_cgraph * g = st.g;
+    const ggml_tensor * n = g->nodes[i];
+    if (i + 2 >= g->n_nodes || st.done[i + 1] || st.done[i + 2]) return 0;
+    const ggml_tensor * y = n->src[0], * b = n->src[1];
+    const ggml_tensor * n1 = g->nodes[i + 1], * n2 = g->nodes[i + 2];
+    if (n1->op != GGML_OP_ADD || n2->op != GGML_OP_ADD || !is_f32_contig(n) || !is_f32_contig(y) || !same_shape(n, y) || !is_row_of(b, n) || n->ne[1] * n->ne[2] * n->ne[3] < 1) return 0;
+    const ggml_tensor * a = n1->src[0] == n ? n1->src[1] : (n1->src[1] == n ? n1->src[0] : nullptr);
+    const ggml_tensor * x = n2->src[0] == n1 ? n2->src[1] : (n2->src[1] == n1 ? n2->src[0] : nullptr);
+    if (!a || !x || a == n || x == n1 || !is_f32_contig(a) || !is_f32_contig(x) || !same_shape(a, n) || !same_shape(x, n) || !is_f32_contig(n1) || !is_f32_contig(n2) ||
+        !same_shape(n1, n) || !same_shape(n2, n) || !single_use(st, n) || !single_use(st, n1)) return 0;
+    if (!elementwise_safe(n2, x) || !elementwise_safe(n2, a) || !elementwise_safe(n2, y) || ranges_overlap(n2, b)) return 0;
+    launch_add_chain(st.c->stream, (const float *) x->data, (const float *) a->data, (const float *) y->data, (const float *) b->data, (float *) n2->data, n->ne[0], ggml_abi_nrows(n));
+    st.c->st.kernel_launches++;
+    st.c->st.fused_nodes += 2;
+    return 3;
+}
+
+// ROPE over a frequency table, rotate-half over the whole row: the shapes the two fusions below serve
+static bool rope_table_plain(const ggml_tensor * n) {
+    const ggml_tensor * a = n->src[0];
+    return n->op_params[3] == 2 && n->src[2] && (n->op_params[2] == GGML_ROPE_TYPE_NEOX) && n->op_params[1] == a->ne[0] && (a->ne[0] % 2) == 0 && a->type == GGML_TYPE_F32 && a->nb[0] == 4 &&
+           n->type == GGML_TYPE_F32 && n->ne[3] == 1 && n->src[1]->type == GGML_TYPE_I32 && n->src[2]->type == GGML_TYPE_F32 && ggml_abi_is_contiguous(n->src[2]);
+}
+// ROPE(k_r; table) -> RESHAPE -> CONCAT(latent, .; dim 0) -> SET_ROWS(cache): the latent cache row written in place.  Returns the nodes consumed
+static int try_fuse_latent_row_store(exec_state & st, int i) {
+    ggml_cgraph * g = st.g;
+    const ggml_tensor * n = g->nodes[i];
+    if (i + 3 >= g->n_nodes || st.done[i + 1] || st.done[i + 2] || st.done[i + 3] || !rope_table_plain(n) || n->ne[1] != 1) return 0;
+    const ggml_tensor * rs = g->nodes[i + 1], * cc = g->nodes[i + 2], * sr = g->nodes[i + 3];
+    if (rs->op != GGML_OP_RESHAPE || rs->src[0] != n || cc->op != GGML_OP_CONCAT || cc->op_params[0] != 0 || cc->src[1] != rs || sr->op != GGML_OP_SET_ROWS || sr->src[0] != cc) return 0;
+    const ggml_tensor * lat = cc->src[0], * idx = sr->src[1];
+    const int64_t T = n->ne[2];
+    if (lat->type != GGML_TYPE_F32 || lat->nb[0] != 4 || lat->ne[1] != T || lat->ne[2] != 1 || lat->ne[3] != 1 || idx->type != GGML_TYPE_I64 || !ggml_abi_is_contiguous(idx) || ggml_abi_nelements(idx) != T) return 0;
+    if (!(sr->type == GGML_TYPE_F32 || sr->type == GGML_TYPE_BF16 || sr->type == GGML_TYPE_F16) || sr->nb[0] != ggml_abi_type_size(sr->type) || sr->ne[0] != lat->ne[0] + n->ne[0]) return 0;
+    if (!single_use(st, n) || !single_use(st, rs) || !single_use(st, cc)) return 0;
+    launch_latent_row_store(st.c->stream, TD(lat), TD(n->src[0]), TD(n->src[1]), (const float *) n->src[2]->data, ggml_abi_op_param_f32(n, 8), (int) n->ne[0], (const int64_t *) idx->data, TD(sr));
+    st.c->st.kernel_launches++;
+    st.c->st.fused_nodes += 3;
+    return 4;
+}
+// ROPE(q_r; table) -> CONCAT(q in the latent space, .; dim 0): the query rows in one launch.  Returns the nodes consumed
+static int try_fuse_concat_rope(exec_state & st, int i) {
+    ggml_cgraph * g = st.g;
+    const ggml_tensor * n = g->nodes[i];
+    if (i + 1 >= g->n_nodes || st.done[i + 1] || !rope_table_plain(n)) return 0;
+    const ggml_tensor * cc = g->nodes[i + 1];
+    if (cc->op != GGML_OP_CONCAT || cc->op_params[0] != 0 || cc->src[1] != n || !single_use(st, n) || !is_f32_contig(cc)) return 0;
+    const ggml_tensor * qa = cc->src[0];
+    if (qa->type != GGML_TYPE_F32 || qa->nb[0] != 4 || qa->ne[1] != n->ne[1] || qa->ne[2] != n->ne[2] || qa->ne[3] != 1 || ranges_overlap(cc, qa) || ranges_overlap(cc, n->src[0])) return 0;
+    launch_concat_rope(st.c->stream, TD(qa), TD(n->src[0]), TD(n->src[1]), (const float *) n->src[2]->data, ggml_abi_op_param_f32(n, 8), TD(cc));
+    st.c->st.kernel_launches++;
+    st.c->st.fused_nodes += 1;
+    return 2;
+}
+
 static int run_node(exec_state & st, int i) {
     backend_ctx * c = st.c;
     ggml_cgraph * g = st.g;
@@ -2045,12 +2174,24 @@ static int run_node(exec_state & st, int i) {
                 const int used = try_fuse_expert_sum(st, i);
                 if (used > 0) return used;
             }
+            static const bool row_fusions = !getenv("GGML_MI355X_ROW_FUSIONS") || atoi(getenv("GGML_MI355X_ROW_FUSIONS")) != 0;
+            if (fuse && row_fusions && n->op == GGML_OP_ADD && a->op == GGML_OP_MUL_MAT) {
+                if (try_fuse_geglu_bias(st, i)) return 1;
+                const int used = try_fuse_add_chain(st, i);
+                if (used > 0) return used;
+            }
             timed_scope ts(c, "binary", (double) ggml_abi_nbytes(n) * 3);
             launch_binary(s, n->op, TD(a), TD(b), TD(n));
             c->st.kernel_launches++;
             return 1;
         }
         case GGML_OP_CONCAT: {
+            static const bool row_fusions = !getenv("GGML_MI355X_ROW_FUSIONS") || atoi(getenv("GGML_MI355X_ROW_FUSIONS")) != 0;
+            if (fuse && row_fusions) {
+                timed_scope ts(c, "token_shift", (double) ggml_abi_nbytes(a) * 3);
+                const int used = try_fuse_token_shift(st, i);
+                if (used > 0) return used;
+            }
             timed_scope ts(c, "concat", (double) ggml_abi_nbytes(n) * 2);
             launch_concat(s, TD(a), TD(b), TD(n), n->op_params[0]);
             c->st.kernel_launches++;
@@ -2081,6 +2222,20 @@ static int run_node(exec_state & st, int i) {
             return 1;
         }
         case GGML_OP_UNARY: {
+            // SIGMOID(g) -> RESHAPE -> MUL(x, .) with ONE gate per row of x (a number per head): one pass
+            if (fuse && n->op_params[0] == GGML_UNARY_OP_SIGMOID && next(1) && next(2) && !st.done[i + 1] && !st.done[i + 2]) {
+                const ggml_tensor * rs = next(1), * gm2 = next(2);
+                if (rs->op == GGML_OP_RESHAPE && rs->src[0] == n && rs->ne[0] == 1 && gm2->op == GGML_OP_MUL && gm2->src[1] == rs && single_use(st, n) && single_use(st, rs)) {
+                    const ggml_tensor * x = gm2->src[0];
+                    if (is_f32_contig(x) && is_f32_contig(gm2) && same_shape(x, gm2) && is_f32_contig(a) && ggml_abi_nelements(a) == ggml_abi_nrows(x) && rs->ne[1] == x->ne[1] && rs->ne[2] == x->ne[2] &&
+                        elementwise_safe(gm2, x) && !ranges_overlap(gm2, a)) {
+                        launch_mul_sigmoid_rows(s, (const float *) x->data, (const float *) a->data, (float *) gm2->data, x->ne[0], ggml_abi_nrows(x));
+                        c->st.kernel_launches++;
+                        c->st.fused_nodes += 2;
+                        return 3;
+                    }
+                }
+            }
             // SIGMOID(g) -> MUL(x, sigmoid): a gate in one pass
             ggml_tensor * gm = next(1);
             if (fuse && n->op_params[0] == GGML_UNARY_OP_SIGMOID && gm && gm->op == GGML_OP_MUL && (gm->src[0] == n || gm->src[1] == n) && gm->src[0] != gm->src[1] && single_use(st, n)) {
@@ -2253,6 +2408,19 @@ static int run_node(exec_state & st, int i) {
             return 1;
         }
         case GGML_OP_GET_ROWS: {
+            // GET_ROWS(x, rows) -> SET_ROWS(state, ., slots), f32 to f32: chosen rows copied straight to their destination rows
+            if (fuse && next(1) && !st.done[i + 1] && next(1)->op == GGML_OP_SET_ROWS && next(1)->src[0] == n && single_use(st, n)) {
+                const ggml_tensor * sr = next(1);
+                const ggml_tensor * di = sr->src[1];
+                if (a->type == GGML_TYPE_F32 && a->nb[0] == 4 && n->ne[2] == 1 && n->ne[3] == 1 && b->type == GGML_TYPE_I32 && ggml_abi_is_contiguous(b) && sr->type == GGML_TYPE_F32 && sr->nb[0] == 4 &&
+                    sr->ne[0] == a->ne[0] && di->type == GGML_TYPE_I64 && ggml_abi_is_contiguous(di) && ggml_abi_nelements(di) == n->ne[1] && ggml_abi_nelements(b) == n->ne[1] && !ranges_overlap(sr, a)) {
+                    timed_scope ts(c, "copy_rows", (double) ggml_abi_nbytes(n) * 2);
+                    launch_copy_rows_indexed(s, TD(a), (const int32_t *) b->data, (const int64_t *) di->data, n->ne[1], TD(sr));
+                    c->st.kernel_launches++;
+                    c->st.fused_nodes++;
+                    return 2;
+                }
+            }
             // the head of a decode step (round 6): the token embeddings' GET_ROWS, the mask's F32 -> F16 cast (an input leaf cast once per graph) and the (cos, sin) table
             // the fused Q/K/V launches of every layer read are independent of each other — one launch instead of three at the dependent-launch floor.  The cast is
             // hoisted over the nodes between only when its result's memory is not touched by any of them; the table is the one ensure_rope_table would build at the
@@ -2399,6 +2567,12 @@ static int run_node(exec_state & st, int i) {
             return 1;
         }
         case GGML_OP_ROPE: {
+            if (fuse && n->op_params[3] == 2) {
+                timed_scope ts(c, "rope_rows", (double) ggml_abi_nbytes(n) * 2);
+                int used = try_fuse_latent_row_store(st, i);
+                if (used == 0) used = try_fuse_concat_rope(st, i);
+                if (used > 0) return used;
+            }
             if (fuse && try_fuse_rope_store(st, i)) return 1;
             static const bool row_stores = !getenv("GGML_MI355X_ROW_STORES") || atoi(getenv("GGML_MI355X_ROW_STORES")) != 0;
             if (fuse && row_stores && n->type == GGML_TYPE_F32 && a->type == GGML_TYPE_F32 && a->nb[0] == 4 && !(n->op_params[2] & GGML_ROPE_TYPE_MROPE) && !n->src[2] && n->ne[3] == 1 &&

@@ -251,6 +251,14 @@ void launch_rms_norm_mul_quantize(hipStream_t s, const tdesc & x, const float * 
 void launch_swiglu_quantize(hipStream_t s, const tdesc & a, const tdesc * b, int64_t nc, int swapped, void * dst_q8k);
 void launch_cpy(hipStream_t s, const tdesc & src, const tdesc & dst);
 void launch_concat(hipStream_t s, const tdesc & a, const tdesc & b, const tdesc & dst, int dim);  // f32, any strides
+// fused steps of models with token shift / latent attention (ops.hip): each is the arithmetic of the nodes it replaces, operation by operation
+void launch_token_shift(hipStream_t s, const float * h, int64_t n, int64_t n_tok, const tdesc & state, const int32_t * src, const float * w, float * out);
+void launch_copy_rows_indexed(hipStream_t s, const tdesc & a, const int32_t * src_idx, const int64_t * dst_idx, int64_t n_rows, const tdesc & d);
+void launch_geglu_bias(hipStream_t s, const float * g, const float * bg, const float * u, const float * bu, float * d, int64_t n, int64_t rows);
+void launch_add_chain(hipStream_t s, const float * x, const float * a, const float * y, const float * b, float * d, int64_t n, int64_t rows);
+void launch_mul_sigmoid_rows(hipStream_t s, const float * x, const float * g, float * d, int64_t n, int64_t rows);
+void launch_latent_row_store(hipStream_t s, const tdesc & lat, const tdesc & kr, const tdesc & pos, const float * freq, float mag, int n_rot, const int64_t * idx, const tdesc & cache);
+void launch_concat_rope(hipStream_t s, const tdesc & a, const tdesc & b, const tdesc & pos, const float * freq, float mag, const tdesc & d);
 void launch_get_rows(hipStream_t s, const tdesc & src, const tdesc & idx, const tdesc & dst);
 void launch_set_rows(hipStream_t s, const tdesc & src, const tdesc & idx, const tdesc & dst);
 void launch_cpy_q8_0(hipStream_t s, const void * src, void * dst, int64_t n_values, bool to_q8);  // contiguous Q8_0 <-> F32 (K-shift of a quantised cache)

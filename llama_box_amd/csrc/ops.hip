@@ -1091,6 +1091,126 @@ void launch_rope_store(hipStream_t s, const tdesc & a, const tdesc & pos, const 
     rope_host_consts(p, theta_scale, c0, c1);
     hipLaunchKernelGGL(k_rope_store, dim3((unsigned) a.ne[1], (unsigned) a.ne[2]), dim3(64), 0, s, a, pos, ff, idx, cache.data, cache.nb[1], cache.type, p, theta_scale, c0, c1);
 }
+// ------------------------------------------------------------------------------------------------ fused steps of models with token shift / latent attention
+// (each one the arithmetic of the unfused nodes it replaces, operation by operation: fused and unfused graphs agree bit for bit)
+// token shift: out[t] = h[t] + (prev - h[t]) * w, prev = row src[t] of [h rows | state rows] (CONCAT dim 1 -> GET_ROWS -> SUB -> MUL -> ADD)
+__global__ void __launch_bounds__(256) k_token_shift(const float * __restrict__ h, const int64_t n, const int64_t n_tok, const char * __restrict__ state, const int64_t state_nb1,
+                                                     const int32_t * __restrict__ src, const float * __restrict__ w, float * __restrict__ out) {
+    const int64_t t = blockIdx.x;
+    const int64_t r = src[t];
+    const float * __restrict__ prev = r < n_tok ? h + r * n : (const float *) (state + (r - n_tok) * state_nb1);
+    const float * __restrict__ cur = h + t * n;
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+        const float x = cur[i];
+        const float d = prev[i] - x;
+        const float m = d * w[i];
+        out[t * n + i] = x + m;
+    }
+}
+void launch_token_shift(hipStream_t s, const float * h, int64_t n, int64_t n_tok, const tdesc & state, const int32_t * src, const float * w, float * out) {
+    if (n_tok == 0) return;
+    hipLaunchKernelGGL(k_token_shift, dim3((unsigned) n_tok), dim3(256), 0, s, h, n, n_tok, state.data, state.nb[1], src, w, out);
+}
+// rows src_idx[r] of a (f32) copied to rows dst_idx[r] of d (f32): GET_ROWS -> SET_ROWS (a sequence's last row of a batch becomes its state row)
+__global__ void __launch_bounds__(256) k_copy_rows_indexed(const tdesc a, const int32_t * __restrict__ src_idx, const int64_t * __restrict__ dst_idx, const tdesc d) {
+    const int64_t r = blockIdx.x;
+    const float * __restrict__ x = (const float *) (a.data + (int64_t) src_idx[r] * a.nb[1]);
+    float * __restrict__ y = (float *) (d.data + dst_idx[r] * d.nb[1]);
+    for (int64_t i = threadIdx.x; i < a.ne[0]; i += blockDim.x) y[i] = x[i];
+}
+void launch_copy_rows_indexed(hipStream_t s, const tdesc & a, const int32_t * src_idx, const int64_t * dst_idx, int64_t n_rows, const tdesc & d) {
+    if (n_rows == 0) return;
+    hipLaunchKernelGGL(k_copy_rows_indexed, dim3((unsigned) n_rows), dim3(256), 0, s, a, src_idx, dst_idx, d);
+}
+// gated tanh-GELU with biases: d = gelu(g + bg) * (u + bu) (ADD, ADD, UNARY GELU, MUL); rows of n values
+__global__ void __launch_bounds__(256) k_geglu_bias(const float * __restrict__ g, const float * __restrict__ bg, const float * __restrict__ u, const float * __restrict__ bu,
+                                                    float * __restrict__ d, const int64_t n, const int64_t total) {
+    for (int64_t e = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (int64_t) gridDim.x * blockDim.x) {
+        const int64_t i = e % n;
+        const float v = g[e] + bg[i];
+        const float a = 0.5f * v * (1.0f + tanhf(0.79788456080286535588f * (v + 0.044715f * v * v * v)));
+        const float b = u[e] + bu[i];
+        d[e] = a * b;
+    }
+}
+void launch_geglu_bias(hipStream_t s, const float * g, const float * bg, const float * u, const float * bu, float * d, int64_t n, int64_t rows) {
+    const int64_t total = n * rows;
+    if (total == 0) return;
+    hipLaunchKernelGGL(k_geglu_bias, dim3((unsigned) std::min<int64_t>((total + 255) / 256, 4096)), dim3(256), 0, s, g, bg, u, bu, d, n, total);
+}
+// d = x + (a + (y + b)): a projection's bias, the sum of two parallel sublayers and the residual (ADD, ADD, ADD); b is a row of n values, or absent
+__global__ void __launch_bounds__(256) k_add_chain(const float * __restrict__ x, const float * __restrict__ a, const float * __restrict__ y, const float * __restrict__ b,
+                                                   float * __restrict__ d, const int64_t n, const int64_t total) {
+    for (int64_t e = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (int64_t) gridDim.x * blockDim.x) {
+        const float yb = b ? y[e] + b[e % n] : y[e];
+        const float s2 = a[e] + yb;
+        d[e] = x[e] + s2;
+    }
+}
+void launch_add_chain(hipStream_t s, const float * x, const float * a, const float * y, const float * b, float * d, int64_t n, int64_t rows) {
+    const int64_t total = n * rows;
+    if (total == 0) return;
+    hipLaunchKernelGGL(k_add_chain, dim3((unsigned) std::min<int64_t>((total + 255) / 256, 4096)), dim3(256), 0, s, x, a, y, b, d, n, total);
+}
+// heads gated by ONE number each: d[r][i] = x[r][i] * sigmoid(g[r]) (UNARY SIGMOID -> MUL with the gate broadcast over a head's entries)
+__global__ void __launch_bounds__(256) k_mul_sigmoid_rows(const float * __restrict__ x, const float * __restrict__ g, float * __restrict__ d, const int64_t n, const int64_t total) {
+    for (int64_t e = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (int64_t) gridDim.x * blockDim.x) {
+        const float sg = 1.f / (1.f + expf(-g[e / n]));
+        d[e] = x[e] * sg;
+    }
+}
+void launch_mul_sigmoid_rows(hipStream_t s, const float * x, const float * g, float * d, int64_t n, int64_t rows) {
+    const int64_t total = n * rows;
+    if (total == 0) return;
+    hipLaunchKernelGGL(k_mul_sigmoid_rows, dim3((unsigned) std::min<int64_t>((total + 255) / 256, 4096)), dim3(256), 0, s, x, g, d, n, total);
+}
+// a latent cache row: [lat[t] (n_lat values) | rotate-half(kr[t]) (n_rot values, frequency table)] stored as row idx[t] of the cache in its type
+// (ROPE -> CONCAT dim 0 -> SET_ROWS)
+__global__ void __launch_bounds__(128) k_latent_row_store(const tdesc lat, const tdesc kr, const tdesc pos, const float * __restrict__ freq, const float mag, const int n_rot,
+                                                          const int64_t * __restrict__ idx, char * __restrict__ cache, const int64_t cache_nb1, const int cache_type) {
+    const int64_t t = blockIdx.x;
+    const int64_t n_lat = lat.ne[0];
+    const float * __restrict__ l = (const float *) (lat.data + t * lat.nb[1]);
+    const float * __restrict__ r = (const float *) (kr.data + t * kr.nb[2]);
+    char * __restrict__ row = cache + idx[t] * cache_nb1;
+    for (int64_t i = threadIdx.x; i < n_lat; i += blockDim.x) store_as(row, cache_type, i, l[i]);
+    const float pos_f = (float) *(const int32_t *) (pos.data + t * pos.nb[0]);
+    const int half = n_rot / 2;
+    for (int ip = threadIdx.x; ip < half; ip += blockDim.x) {
+        float cs, sn;
+        rope_cos_sin_table(ip, pos_f, freq, mag, cs, sn);
+        const float x0 = r[ip], x1 = r[ip + half];
+        store_as(row, cache_type, n_lat + ip, x0 * cs - x1 * sn);
+        store_as(row, cache_type, n_lat + ip + half, x0 * sn + x1 * cs);
+    }
+}
+void launch_latent_row_store(hipStream_t s, const tdesc & lat, const tdesc & kr, const tdesc & pos, const float * freq, float mag, int n_rot, const int64_t * idx, const tdesc & cache) {
+    if (lat.ne[1] == 0) return;
+    hipLaunchKernelGGL(k_latent_row_store, dim3((unsigned) lat.ne[1]), dim3(128), 0, s, lat, kr, pos, freq, mag, n_rot, idx, cache.data, cache.nb[1], cache.type);
+}
+// the query rows of latent attention: d[.., h, t] = [a[.., h, t] (n_a values, any strides) | rotate-half(b[.., h, t]) (n_rot values, frequency table)] (ROPE -> CONCAT dim 0)
+__global__ void __launch_bounds__(128) k_concat_rope(const tdesc a, const tdesc b, const tdesc pos, const float * __restrict__ freq, const float mag, const tdesc d) {
+    const int64_t h = blockIdx.x, t = blockIdx.y;
+    const int64_t n_a = a.ne[0];
+    const int half = (int) (b.ne[0] / 2);
+    const float * __restrict__ x = (const float *) (a.data + h * a.nb[1] + t * a.nb[2]);
+    const float * __restrict__ r = (const float *) (b.data + h * b.nb[1] + t * b.nb[2]);
+    float * __restrict__ out = (float *) (d.data + h * d.nb[1] + t * d.nb[2]);
+    for (int64_t i = threadIdx.x; i < n_a; i += blockDim.x) out[i] = x[i];
+    const float pos_f = (float) *(const int32_t *) (pos.data + t * pos.nb[0]);
+    for (int ip = threadIdx.x; ip < half; ip += blockDim.x) {
+        float cs, sn;
+        rope_cos_sin_table(ip, pos_f, freq, mag, cs, sn);
+        const float x0 = r[ip], x1 = r[ip + half];
+        out[n_a + ip] = x0 * cs - x1 * sn;
+        out[n_a + ip + half] = x0 * sn + x1 * cs;
+    }
+}
+void launch_concat_rope(hipStream_t s, const tdesc & a, const tdesc & b, const tdesc & pos, const float * freq, float mag, const tdesc & d) {
+    if (d.ne[1] * d.ne[2] == 0) return;
+    hipLaunchKernelGGL(k_concat_rope, dim3((unsigned) d.ne[1], (unsigned) d.ne[2]), dim3(128), 0, s, a, b, pos, freq, mag, d);
+}
+
 // a x + b y (k_axpby's arithmetic) stored as rows of a cache: row t of n values goes to cache row idx[t]
 __global__ void __launch_bounds__(256) k_axpby_store(const float * __restrict__ x, const float a, const float * __restrict__ y, const float b, const int64_t n, const int64_t * __restrict__ idx,
                                                      char * __restrict__ cache, const int64_t cache_nb1, const int cache_type) {

@@ -228,6 +228,26 @@ def test_greedy_generation_through_the_engine(backend, tmp_path, H):
     s.free()
 
 
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_fused_steps_equal_the_unfused_nodes(backend, tmp_path, dtype):
+    """token shift, state rows, gated activation with biases, bias + sublayer sum + residual, head gates, latent cache rows and query rows as single launches: bit for bit
+    what the graph's own nodes give, for a prompt portion and for single tokens"""
+    cfg = cfg_a()
+    t = toks(90, cfg["vocab"], 41)
+    rows = {}
+    launches = {}
+    for fusion in (1, 0):
+        backend.set_option("fusion", fusion)
+        s = Served(backend, tmp_path / str(fusion), cfg, 18, dtype)
+        before = backend.stat("kernel_launches")
+        rows[fusion] = np.concatenate([s.feed("x", t[:70])] + [s.feed("x", [tok]) for tok in t[70:]])
+        launches[fusion] = backend.stat("kernel_launches") - before
+        s.free()
+    backend.set_option("fusion", 1)
+    assert np.array_equal(rows[0], rows[1])
+    assert launches[1] < 0.7 * launches[0]
+
+
 # ------------------------------------------------------------------------------------------------ edges: the data must show a rule that is one off
 def _variant(cfg, il, **mask):
     c = copy.deepcopy(cfg)
