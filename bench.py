@@ -202,7 +202,8 @@ def bench_nigozen(args):
         rng = np.random.default_rng(1)
         prompt = rng.integers(0, n_vocab, n_prompt).tolist()
         res = {}
-        for rep in range(2):  # the first pass warms up (graph capture, scratch growth)
+        best_p, best_d = None, None
+        for rep in range(2 if not args.zigipel else 4):  # the first pass warms up (graph capture, scratch growth); the Zigipel comparison keeps the best of the three that follow
             ctx.clear()
             be.synchronize()
             t0 = time.perf_counter()
@@ -213,7 +214,11 @@ def bench_nigozen(args):
                 rc, _ = ctx.decode([prompt[i]], [n_prompt + i], copy_logits=False)
                 assert rc == 0
             t2 = time.perf_counter()
-            res = {"prefill_tok_s": round(n_prompt / (t1 - t0), 1), "decode_tok_s": round(n_dec / (t2 - t1), 1), "prefill_ms": round((t1 - t0) * 1e3, 2), "decode_ms_per_tok": round((t2 - t1) * 1e3 / n_dec, 3)}
+            if rep > 0:
+                best_p = (t1 - t0) if best_p is None or not args.zigipel else min(best_p, t1 - t0)
+                best_d = (t2 - t1) if best_d is None or not args.zigipel else min(best_d, t2 - t1)
+        if True:
+            res = {"prefill_tok_s": round(n_prompt / best_p, 1), "decode_tok_s": round(n_dec / best_d, 1), "prefill_ms": round(best_p * 1e3, 2), "decode_ms_per_tok": round(best_d * 1e3 / n_dec, 3)}
         if os.environ.get("BENCH_NIGOZEN_CLASSES", "1") == "0":  # (a run under a profiler: its own kernel trace replaces the event-bracketed pass)
             ctx.free()
             return res
@@ -236,22 +241,23 @@ def bench_nigozen(args):
     if args.zigipel:  # Zigipel beside Nigozen (all layers dense) with as many layers as Zigipel has layer runs, equal width, heads, head size and vocabulary
         out["metric"] = "zigipel_vs_nigozen_tokens_per_s"
         out["dtype"] = "bf16 (both)"
+        be.close()
         for name in args.zigipel.split(","):
             z = ZIGIPEL_SIZES[name]
-            mz = Model(config_json=_json.dumps(zigipel_config(z)), seed=7, buft=be.buft, wtype=L.BF16)
-            r_z = run(mz, z["vocab"])
-            r_z["weight_bytes"] = int(L.host().llm_model_total_bytes(mz.m))
-            r_z["stream_bytes_per_token"] = mz.stream_bytes()
-            mz.free()
             zn = dict(width=z["width"], layers=6, heads=z["heads"], kv=z["kv"], hd=z["hd"], rot=z["hd"] // 2, chunk=z["window"], ff=z["ff"] * 3 // 2, vocab=z["vocab"])
-            mn = Model(config_json=_json.dumps(nigozen_config(zn, dense_only=True)), seed=7, buft=be.buft, wtype=L.BF16)
-            r_n = run(mn, z["vocab"])
-            r_n["stream_bytes_per_token"] = mn.stream_bytes()
-            mn.free()
-            out["sizes"][name] = {"config": z, "zigipel": r_z, "nigozen_dense": r_n, "prefill_ratio": round(r_z["prefill_tok_s"] / r_n["prefill_tok_s"], 3),
-                                  "decode_ratio": round(r_z["decode_tok_s"] / r_n["decode_tok_s"], 3)}
+            res = {}
+            for side, cfg in (("zigipel", zigipel_config(z)), ("nigozen_dense", nigozen_config(zn, dense_only=True))):
+                be = L.Backend(0)  # (a backend of its own per model: the event-bracketed pass of one model leaves nothing behind for the next one's timed run)
+                mdl = Model(config_json=_json.dumps(cfg), seed=7, buft=be.buft, wtype=L.BF16)
+                res[side] = run(mdl, z["vocab"])
+                res[side]["weight_bytes"] = int(L.host().llm_model_total_bytes(mdl.m))
+                res[side]["stream_bytes_per_token"] = mdl.stream_bytes()
+                mdl.free()
+                be.close()
+            out["sizes"][name] = {"config": z, "zigipel": res["zigipel"], "nigozen_dense": res["nigozen_dense"],
+                                  "prefill_ratio": round(res["zigipel"]["prefill_tok_s"] / res["nigozen_dense"]["prefill_tok_s"], 3),
+                                  "decode_ratio": round(res["zigipel"]["decode_tok_s"] / res["nigozen_dense"]["decode_tok_s"], 3)}
         print(_json.dumps(out))
-        be.close()
         return
     for name in args.nigozen.split(","):
         z = NIGOZEN_SIZES[name]

@@ -93,6 +93,7 @@ __global__ void __launch_bounds__(256) k_attn_f32_rows(const tdesc q, const tdes
     const char * vbase = v.data + g * v.nb[2];
     const bool pen = r12 != nullptr;
     const float r1 = pen ? r12[h] : 0.0f, r2 = pen ? r12[q.ne[2] + h] : 0.0f;
+    const bool k_vec = KT != GGML_TYPE_F32 && (DK % 8) == 0 && (k.nb[1] % 16) == 0 && (k.nb[2] % 16) == 0 && (((uintptr_t) k.data) & 15) == 0;
     float m = ATTN_F32_LOW, l = 0.0f;
     if (sinks && wave == 0) { m = sinks[h]; l = 1.0f; }  // the sink: exp(sink - m) = 1 in the denominator, nothing in the numerator
     float acc[ATTN_F32_MAX_D / 64];
@@ -109,6 +110,23 @@ __global__ void __launch_bounds__(256) k_attn_f32_rows(const tdesc q, const tdes
         if (vis) {
             const char * krow = kbase + j * k.nb[1];
             float d = 0.0f;
+            if constexpr (KT != GGML_TYPE_F32) {
+                if (k_vec) {  // 16-byte loads of eight 2-byte values; the sum runs over i in the same order as the scalar loop below
+                    for (int i = 0; i < DK; i += 8) {
+                        const uint4 w = *(const uint4 *) (krow + i * 2);
+                        const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            float lo, hi;
+                            if constexpr (KT == GGML_TYPE_BF16) { lo = __uint_as_float(u[e] << 16); hi = __uint_as_float(u[e] & 0xFFFF0000u); }
+                            else { lo = h2f((uint16_t) (u[e] & 0xFFFFu)); hi = h2f((uint16_t) (u[e] >> 16)); }
+                            d = fmaf(qs[i + 2 * e], lo, d);
+                            d = fmaf(qs[i + 2 * e + 1], hi, d);
+                        }
+                    }
+                } else
+                for (int i = 0; i < DK; ++i) d = fmaf(qs[i], kv_ld<KT>(krow, i), d);
+            } else
             for (int i = 0; i < DK; ++i) d = fmaf(qs[i], kv_ld<KT>(krow, i), d);
             s = d * scale + mask_term(mv, pen, r1, r2);
         }
