@@ -442,6 +442,186 @@ __global__ void __launch_bounds__(256) k_attn_mma_bf16(const tdesc q, const tdes
                 for (int r = 0; r < 4; ++r) if (d0 + r < DV) out[d0 + r] = O[dt][4 * b + r] * inv;
         }
 }
+// k_attn_mma_bf16_wide: the same scheme for ONE key/value head shared by all query heads and rows wider than a wave can hold — a latent cache row [latent | rotated part] of
+// several hundred values, its leading part the value.  The queries of a workgroup are 32 (token, head) pairs (head fastest); its four waves share them: wave w computes the
+// partial scores over a quarter of the key entries, the partials meet in LDS (every wave adds them in the order 0 .. 3 and so holds the same scores), every wave runs the f32
+// soft-max, and wave w accumulates a quarter of the value entries (O^T tiles of 32).  V^T of the block is staged once for all four.  DKQ: 16-entry key groups per wave, DVQ:
+// 32-entry value tiles per wave.
+template <int DKQ, int DVQ>
+__global__ void __launch_bounds__(256) k_attn_mma_bf16_wide(const tdesc q, const tdesc k, const tdesc v, const tdesc mask, const float * __restrict__ sinks, const float * __restrict__ r12,
+                                                            const tdesc dst, const float scale) {
+    constexpr int VS = 36;
+    constexpr int DVT = 4 * DVQ;
+    __shared__ __attribute__((aligned(16))) uint16_t Vt[DVT * 32 * VS];
+    __shared__ float Sp[4][16][64];
+    __shared__ int flag[2];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n = lane & 31, g = lane >> 5;
+    const int64_t H = q.ne[2], n_tok = q.ne[1], n_kv = k.ne[1];
+    const int DK = (int) q.ne[0], DV = (int) v.ne[0];
+    const int64_t qi = (int64_t) blockIdx.x * 32 + n;  // this lane's (token, head) pair
+    const bool q_live = qi < n_tok * H;
+    const int64_t tq = q_live ? qi / H : 0, h = q_live ? qi % H : 0;
+    const char * kbase = k.data;
+    const char * vbase = v.data;
+    uint4 qf[DKQ];
+    {
+        const float * qrow = (const float *) (q.data + tq * q.nb[1] + h * q.nb[2]);
+#pragma unroll
+        for (int s = 0; s < DKQ; ++s) {
+            const int i0 = 16 * (wave * DKQ + s) + 8 * g;
+            uint32_t b[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) b[e] = (q_live && i0 + e < DK) ? att_bf16_bits(qrow[i0 + e]) : 0u;
+            qf[s] = make_uint4(b[0] | (b[1] << 16), b[2] | (b[3] << 16), b[4] | (b[5] << 16), b[6] | (b[7] << 16));
+        }
+    }
+    const bool pen = r12 != nullptr;
+    const float r1 = pen ? r12[h] : 0.0f, r2 = pen ? r12[H + h] : 0.0f;
+    float m = sinks ? sinks[h] : ATTN_F32_LOW, l = sinks ? 1.0f : 0.0f;
+    att_f16v O[DVQ];
+#pragma unroll
+    for (int dt = 0; dt < DVQ; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) O[dt][i] = 0.0f;
+    const char * mrow = mask.data + tq * mask.nb[1];
+    if (threadIdx.x < 2) flag[threadIdx.x] = 0;
+    __syncthreads();
+    auto load_mask = [&](const int64_t j0, float (&mv)[16]) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int64_t j = j0 + 8 * b + 4 * g;
+            float4 t = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+            if (q_live && j + 3 < n_kv) t = *(const float4 *) (mrow + j * 4);
+            else if (q_live) {
+                if (j < n_kv) t.x = ((const float *) mrow)[j];
+                if (j + 1 < n_kv) t.y = ((const float *) mrow)[j + 1];
+                if (j + 2 < n_kv) t.z = ((const float *) mrow)[j + 2];
+            }
+            mv[4 * b] = t.x; mv[4 * b + 1] = t.y; mv[4 * b + 2] = t.z; mv[4 * b + 3] = t.w;
+        }
+    };
+    float mv_next[16];
+    load_mask(0, mv_next);
+    for (int64_t j0 = 0, blk = 0; j0 < n_kv; j0 += 32, ++blk) {
+        float mv[16];
+        bool any = false;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { mv[i] = mv_next[i]; any = any || mv[i] > -INFINITY; }
+        if (j0 + 32 < n_kv) load_mask(j0 + 32, mv_next);
+        const bool wave_any = __ballot(any) != 0;  // (the four waves hold the same queries: the same answer in each)
+        if (threadIdx.x == 0) flag[(blk + 1) & 1] = 0;
+        if (wave_any && lane == 0) flag[blk & 1] = 1;
+        __syncthreads();
+        if (!flag[blk & 1]) continue;
+        // this wave's quarter of the block's key entries, straight from the cache rows
+        uint4 kf[DKQ];
+        {
+            const int64_t cell = j0 + n < n_kv ? j0 + n : n_kv - 1;
+            const char * krow = kbase + cell * k.nb[1] + g * 16;
+#pragma unroll
+            for (int s = 0; s < DKQ; ++s) {
+                const int sg = wave * DKQ + s;
+                kf[s] = make_uint4(0, 0, 0, 0);
+                if (16 * sg + 8 * g < DK) kf[s] = *(const uint4 *) (krow + sg * 32);
+            }
+        }
+        // V^T of the block (all value entries) into LDS, as in k_attn_mma_bf16
+        for (int e0 = threadIdx.x; e0 < 8 * (DVT * 4); e0 += 256) {
+            const int cg = e0 / (DVT * 4), c8 = e0 % (DVT * 4);
+            uint32_t u[4][4];
+#pragma unroll
+            for (int cc = 0; cc < 4; ++cc) {
+                uint4 t = make_uint4(0, 0, 0, 0);
+                if (j0 + 4 * cg + cc < n_kv && 8 * c8 < DV) t = *(const uint4 *) (vbase + (j0 + 4 * cg + cc) * v.nb[1] + c8 * 16);
+                u[cc][0] = t.x; u[cc][1] = t.y; u[cc][2] = t.z; u[cc][3] = t.w;
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint2 lo2 = make_uint2((u[0][e] & 0xFFFFu) | (u[1][e] << 16), (u[2][e] & 0xFFFFu) | (u[3][e] << 16));
+                const uint2 hi2 = make_uint2((u[0][e] >> 16) | (u[1][e] & 0xFFFF0000u), (u[2][e] >> 16) | (u[3][e] & 0xFFFF0000u));
+                *(uint2 *) (Vt + (8 * c8 + 2 * e) * VS + 4 * cg) = lo2;
+                *(uint2 *) (Vt + (8 * c8 + 2 * e + 1) * VS + 4 * cg) = hi2;
+            }
+        }
+        // partial scores over this wave's key entries
+        {
+            att_f16v Sw;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) Sw[i] = 0.0f;
+#pragma unroll
+            for (int s = 0; s < DKQ; ++s) Sw = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(att_bf8, kf[s]), __builtin_bit_cast(att_bf8, qf[s]), Sw, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) Sp[wave][i][lane] = Sw[i];
+        }
+        __syncthreads();
+        att_f16v S;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) S[i] = ((Sp[0][i][lane] + Sp[1][i][lane]) + Sp[2][i][lane]) + Sp[3][i][lane];
+        float mx = ATTN_F32_LOW;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            S[i] = mv[i] > -INFINITY ? S[i] * scale + mask_term(mv[i], pen, r1, r2) : -INFINITY;
+            mx = fmaxf(mx, S[i]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m, mx);
+        const float corr = expf(m - m_new);
+        float ps = 0.0f;
+        uint32_t hi[8], lo[8];
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) {
+            const float p0 = expf(S[i] - m_new), p1 = expf(S[i + 1] - m_new);
+            ps += p0 + p1;
+            const uint32_t h0 = att_bf16_bits(p0), h1 = att_bf16_bits(p1);
+            hi[i >> 1] = h0 | (h1 << 16);
+            lo[i >> 1] = att_bf16_bits(p0 - __uint_as_float(h0 << 16)) | (att_bf16_bits(p1 - __uint_as_float(h1 << 16)) << 16);
+        }
+        ps += __shfl_xor(ps, 32, 64);
+        l = l * corr + ps;
+        m = m_new;
+#pragma unroll
+        for (int dt = 0; dt < DVQ; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) O[dt][i] *= corr;
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            const uint4 ph = make_uint4(hi[4 * s2], hi[4 * s2 + 1], hi[4 * s2 + 2], hi[4 * s2 + 3]);
+            const uint4 pl = make_uint4(lo[4 * s2], lo[4 * s2 + 1], lo[4 * s2 + 2], lo[4 * s2 + 3]);
+#pragma unroll
+            for (int dt = 0; dt < DVQ; ++dt) {
+                const uint16_t * vr = Vt + (32 * (wave * DVQ + dt) + n) * VS + 16 * s2 + 4 * g;
+                const uint2 a0 = *(const uint2 *) vr, a1 = *(const uint2 *) (vr + 8);
+                const uint4 vf = make_uint4(a0.x, a0.y, a1.x, a1.y);
+                O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(att_bf8, vf), __builtin_bit_cast(att_bf8, ph), O[dt], 0, 0, 0);
+                O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(att_bf8, vf), __builtin_bit_cast(att_bf8, pl), O[dt], 0, 0, 0);
+            }
+        }
+    }
+    if (!q_live) return;
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    float * out = (float *) (dst.data + h * dst.nb[1] + tq * dst.nb[2]);
+#pragma unroll
+    for (int dt = 0; dt < DVQ; ++dt)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int d0 = 32 * (wave * DVQ + dt) + 8 * b + 4 * g;
+            if (d0 + 3 < DV) *(float4 *) (out + d0) = make_float4(O[dt][4 * b] * inv, O[dt][4 * b + 1] * inv, O[dt][4 * b + 2] * inv, O[dt][4 * b + 3] * inv);
+            else
+                for (int r = 0; r < 4; ++r) if (d0 + r < DV) out[d0 + r] = O[dt][4 * b + r] * inv;
+        }
+}
+// one key/value head, rows beyond what k_attn_mma_bf16 holds (up to 640 key and 512 value entries), at least 128 (token, head) pairs: a workgroup walks the whole cache for 32
+// pairs, so a decode step's few pairs are better served by the row kernel's workgroup per pair
+static bool attn_mma_bf16_wide_ok(const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const tdesc & dst) {
+    if (!mask || mask->type != GGML_TYPE_F32 || (mask->nb[1] % 16) != 0 || (((uintptr_t) mask->data) & 15)) return false;
+    if (k.type != GGML_TYPE_BF16 || v.type != GGML_TYPE_BF16 || k.ne[2] != 1 || q.ne[1] * q.ne[2] < 128) return false;
+    if ((q.ne[0] % 8) != 0 || (v.ne[0] % 8) != 0 || (q.ne[0] <= 128 && v.ne[0] <= 128) || q.ne[0] > 640 || v.ne[0] > 512) return false;
+    if ((k.nb[1] % 16) || (v.nb[1] % 16) || (((uintptr_t) k.data | (uintptr_t) v.data | (uintptr_t) dst.data) & 15)) return false;
+    if ((dst.nb[1] % 16) || (dst.nb[2] % 16)) return false;
+    return true;
+}
+
 static bool attn_mma_bf16_ok(const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const tdesc & dst) {
     if (!mask || mask->type != GGML_TYPE_F32 || (mask->nb[1] % 16) != 0 || (((uintptr_t) mask->data) & 15)) return false;
     if (k.type != GGML_TYPE_BF16 || v.type != GGML_TYPE_BF16 || q.ne[1] < 32) return false;
@@ -471,6 +651,17 @@ static void attn_f32_launch_t(hipStream_t s, const tdesc & q, const tdesc & k, c
     const int DK = (int) q.ne[0], DV = (int) v.ne[0];
     if constexpr (KT == GGML_TYPE_BF16 && VT == GGML_TYPE_BF16) {
         static const bool mma_on = !getenv("GGML_MI355X_ATTN_MMA") || atoi(getenv("GGML_MI355X_ATTN_MMA")) != 0;
+        if (mma_on && attn_mma_bf16_wide_ok(q, k, v, mask, dst)) {  // one shared key/value head with wide rows (latent attention): four waves per 32 (token, head) pairs
+            const dim3 grid((unsigned) ((n_q * H + 31) / 32));
+            const int dkq = ((DK + 15) / 16 + 3) / 4, dvq = ((DV + 31) / 32 + 3) / 4;  // per wave: 16-entry key groups (<= 10), 32-entry value tiles (<= 4)
+#define MI_ATT_WIDE(A, B) hipLaunchKernelGGL((k_attn_mma_bf16_wide<A, B>), grid, dim3(256), 0, s, q, k, v, *mask, sinks, r12, dst, scale)
+            const int a = dkq <= 3 ? 3 : (dkq <= 5 ? 5 : 10), b = dvq <= 1 ? 1 : (dvq <= 2 ? 2 : 4);
+            if (a == 3 && b == 1) MI_ATT_WIDE(3, 1); else if (a == 3 && b == 2) MI_ATT_WIDE(3, 2); else if (a == 3) MI_ATT_WIDE(3, 4);
+            else if (a == 5 && b == 1) MI_ATT_WIDE(5, 1); else if (a == 5 && b == 2) MI_ATT_WIDE(5, 2); else if (a == 5) MI_ATT_WIDE(5, 4);
+            else if (b == 1) MI_ATT_WIDE(10, 1); else if (b == 2) MI_ATT_WIDE(10, 2); else MI_ATT_WIDE(10, 4);
+#undef MI_ATT_WIDE
+            return;
+        }
         if (mma_on && attn_mma_bf16_ok(q, k, v, mask, dst)) {  // prompt portions over a bf16 cache: the matrix cores
             // waves per workgroup: four share a staged V^T block; two when four would leave most of the chip's 256 CUs without a workgroup (measured at 512 queries x 16
             // heads: 1.87 ms for 16 launches with two waves, 2.12 with four, 1.99 with one)

@@ -321,6 +321,9 @@ def bf16_bits(a):
     (128, 640, 2, 2, 128, 128, 0, 0),    # no window at all: plain causal with distances
     (33, 100, 3, 3, 40, 72, 9, 12),
     (2, 90, 2, 1, 576, 512, 30, 0),      # head sizes of a large latent
+    (40, 300, 4, 1, 576, 512, 100, 0),   # ... in a prompt portion: 160 (token, head) pairs on the wide matrix-core form over a bf16 cache
+    (45, 150, 3, 1, 160, 136, 40, 2),    # a shared head just beyond 128 entries, value rows that are no multiple of 32
+    (9, 777, 16, 1, 320, 256, 500, 0),
 ])
 def test_attention_with_distance_penalty_and_learned_sinks(backend, H, kv_type, n_q, n_kv, heads, kv_heads, dk, dv, size, keep):
     rng = np.random.default_rng(n_q * 1000 + n_kv)
@@ -338,7 +341,8 @@ def test_attention_with_distance_penalty_and_learned_sinks(backend, H, kv_type, 
     scale = 1.0 / np.sqrt(dk)
     if kv_type == L.BF16:
         k, v = R.bf16_round(k).astype(np.float32), R.bf16_round(v).astype(np.float32)
-        if n_q >= 32 and dk % 8 == 0 and dv % 8 == 0 and dk <= 128 and dv <= 128:
+        wide = kv_heads == 1 and n_q * heads >= 128 and (dk > 128 or dv > 128) and dk <= 640 and dv <= 512
+        if dk % 8 == 0 and dv % 8 == 0 and ((n_q >= 32 and dk <= 128 and dv <= 128) or wide):
             q = R.bf16_round(q).astype(np.float32)  # prompt portions over a bf16 cache run on the matrix cores: the queries are rounded to bf16 like every mat-mul operand
 
     def build(g):
