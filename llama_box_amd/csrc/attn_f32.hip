@@ -74,6 +74,37 @@ __device__ __forceinline__ void attn_f32_pv(const float p, const uint64_t live, 
     }
 }
 
+// the same sum for 2-byte value rows of 256 .. 512 entries with a lane owning EIGHT NEIGHBOURING columns (8 lane .. 8 lane + 7): one 16-byte load per cell and lane instead
+// of eight 2-byte ones.  Cells enter every column's sum in the same order as above, so the results are the same bit for bit.
+template <int VT, int CELLS>
+__device__ __forceinline__ void attn_f32_pv8(const float p, const uint64_t live, const char * __restrict__ vbase, const int64_t v_nb1, const int64_t j0, const int64_t n_kv, const int DV,
+                                             const int lane, float (&acc)[ATTN_F32_MAX_D / 64]) {
+    const uint64_t gmask = (1ull << CELLS) - 1ull;
+    const int col = 8 * lane < DV ? 8 * lane : DV - 8;  // (a lane beyond the row's end re-reads the last group; its sums are dropped later)
+    for (int jj0 = 0; jj0 < 64; jj0 += CELLS) {
+        if (!((live >> jj0) & gmask)) continue;
+        uint4 vv[CELLS];
+#pragma unroll
+        for (int u = 0; u < CELLS; ++u) {
+            const int64_t cell = j0 + jj0 + u < n_kv ? j0 + jj0 + u : n_kv - 1;
+            vv[u] = *(const uint4 *) (vbase + cell * v_nb1 + col * 2);
+        }
+#pragma unroll
+        for (int u = 0; u < CELLS; ++u) {
+            const float pj = __shfl(p, jj0 + u, 64);
+            const uint32_t w[4] = {vv[u].x, vv[u].y, vv[u].z, vv[u].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float lo, hi;
+                if constexpr (VT == GGML_TYPE_BF16) { lo = __uint_as_float(w[e] << 16); hi = __uint_as_float(w[e] & 0xFFFF0000u); }
+                else { lo = h2f((uint16_t) (w[e] & 0xFFFFu)); hi = h2f((uint16_t) (w[e] >> 16)); }
+                acc[2 * e] = fmaf(pj, lo, acc[2 * e]);
+                acc[2 * e + 1] = fmaf(pj, hi, acc[2 * e + 1]);
+            }
+        }
+    }
+}
+
 template <int KT, int VT>
 __global__ void __launch_bounds__(256) k_attn_f32_rows(const tdesc q, const tdesc k, const tdesc v, const tdesc mask, const int has_mask, const float * __restrict__ sinks,
                                                        const float * __restrict__ r12, const tdesc dst, const float scale) {
@@ -93,6 +124,8 @@ __global__ void __launch_bounds__(256) k_attn_f32_rows(const tdesc q, const tdes
     const char * vbase = v.data + g * v.nb[2];
     const bool pen = r12 != nullptr;
     const float r1 = pen ? r12[h] : 0.0f, r2 = pen ? r12[q.ne[2] + h] : 0.0f;
+    // (value rows of 256 .. 512 two-byte entries: a lane owns eight neighbouring columns)
+    const bool v_vec8 = VT != GGML_TYPE_F32 && DV > 256 && DV <= 512 && (DV % 8) == 0 && (v.nb[1] % 16) == 0 && (v.nb[2] % 16) == 0 && (((uintptr_t) v.data) & 15) == 0;
     const bool k_vec = KT != GGML_TYPE_F32 && (DK % 8) == 0 && (k.nb[1] % 16) == 0 && (k.nb[2] % 16) == 0 && (((uintptr_t) k.data) & 15) == 0;
     float m = ATTN_F32_LOW, l = 0.0f;
     if (sinks && wave == 0) { m = sinks[h]; l = 1.0f; }  // the sink: exp(sink - m) = 1 in the denominator, nothing in the numerator
@@ -139,15 +172,23 @@ __global__ void __launch_bounds__(256) k_attn_f32_rows(const tdesc q, const tdes
         for (int r = 0; r < ATTN_F32_MAX_D / 64; ++r) acc[r] *= corr;
         // the visible cells' value rows, CELLS at a time with all their loads in flight together: a wave pays one trip to memory per group (measured: 2 us
         // on an otherwise idle chip), so the groups are as large as the registers allow — 32 cells for value sizes up to 128, 16 beyond
+        if constexpr (VT != GGML_TYPE_F32) {
+            if (v_vec8) { attn_f32_pv8<VT, 16>(p, live, vbase, v.nb[1], j0, n_kv, DV, lane, acc); continue; }
+        }
         if (DV <= 128) attn_f32_pv<VT, 32, 2>(p, live, vbase, v.nb[1], j0, n_kv, DV, lane, acc);
         else if (DV <= 256) attn_f32_pv<VT, 16, 4>(p, live, vbase, v.nb[1], j0, n_kv, DV, lane, acc);
         else attn_f32_pv<VT, 8, ATTN_F32_MAX_D / 64>(p, live, vbase, v.nb[1], j0, n_kv, DV, lane, acc);
     }
     if (lane == 0) { part_m[wave] = m; part_l[wave] = l; }
+    if (v_vec8) {
 #pragma unroll
-    for (int r = 0; r < ATTN_F32_MAX_D / 64; ++r) {
-        const int dcol = lane + 64 * r;
-        if (dcol < DV) part_acc[wave][dcol] = acc[r];
+        for (int e = 0; e < 8; ++e) if (8 * lane + e < DV) part_acc[wave][8 * lane + e] = acc[e];
+    } else {
+#pragma unroll
+        for (int r = 0; r < ATTN_F32_MAX_D / 64; ++r) {
+            const int dcol = lane + 64 * r;
+            if (dcol < DV) part_acc[wave][dcol] = acc[r];
+        }
     }
     __syncthreads();
     if (wave != 0) return;
