@@ -2187,7 +2187,7 @@ static int run_node(exec_state & st, int i) {
         }
         case GGML_OP_CONCAT: {
             static const bool row_fusions = !getenv("GGML_MI355X_ROW_FUSIONS") || atoi(getenv("GGML_MI355X_ROW_FUSIONS")) != 0;
-            if (fuse && row_fusions) {
+            if (fuse && row_fusions && n->op_params[0] == 1 && next(1) && next(1)->op == GGML_OP_GET_ROWS && next(1)->src[0] == n) {
                 timed_scope ts(c, "token_shift", (double) ggml_abi_nbytes(a) * 3);
                 const int used = try_fuse_token_shift(st, i);
                 if (used > 0) return used;
